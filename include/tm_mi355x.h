@@ -505,9 +505,9 @@ int tm_gemm_export(const char* path);
  * Norms, attention scores and weights, and the residual sum are fp32 in both.
  * Weight slots (tm_engine_weight_copy, checkpoint bytes: bf16, [out][in]): "embed", "l<i>.norm1", "l<i>.norm2" (with an ff),
  * "l<i>.mix.q|k|v|o", "l<i>.mix.sink" (with a sink), "l<i>.mlp.up|down", "final.norm", "head". */
-enum { TM_MIXER_ATTENTION = 1, TM_MIXER_LATENT = 2 };
+enum { TM_MIXER_ATTENTION = 1, TM_MIXER_LATENT = 2, TM_MIXER_LIGHTNING = 3, TM_MIXER_DELTA = 4 };
 enum { TM_MLP_NONE = 0, TM_MLP_DENSE = 1, TM_MLP_GATED = 2, TM_MLP_MOE = 3 };
-enum { TM_ACT_RELU2 = 0, TM_ACT_GELU_TANH = 1, TM_ACT_SILU = 2 };
+enum { TM_ACT_RELU2 = 0, TM_ACT_GELU_TANH = 1, TM_ACT_SILU = 2, TM_ACT_XIELU = 3 };
 enum { TM_DTYPE_BF16 = 0, TM_DTYPE_F32 = 1 };
 /* Further block forms, mixers and feed-forwards (every switch off at 0: the block above):
  *   one_norm:    both sublayers read norm1(x) (no norm2)
@@ -540,6 +540,30 @@ typedef struct tm_layer_spec {
     float rot_base;
     int   experts, top;
     int   rot_dims; /* how many of the rot_dim channels turn (the first ones; the rest pass unchanged); 0: all */
+    /* post_norm blocks (all off at 0): x <- x + LN1(mixer(x)); x <- x + LN2(ff(x)) -- the sublayers read the stream itself, the layer
+     * norm (mean and variance, weight "norm<i>" and bias "norm<i>.b") is applied to their RESULT.
+     *   attention in such a block: qkv_bias ("mix.q.b" ...), qk_norm_w: per-head RMS norm of queries and keys times "mix.q.norm" /
+     *     "mix.k.norm" [dim] before the rotation; rot_dims > 0: the first rot_dims channels of every query / key head turn, channel i with
+     *     i + rot_dims / 2 by position * rot_base^(-2 i / rot_dims) / rot_scale; window > 0: position i sees j <= i with i - j < window
+     *     or j < keep_first.
+     *   TM_MIXER_LIGHTNING: linear attention with a state per head, S <- decay[head] S + k v^T, o = S^T q, q, k, v = silu of their
+     *     projections; the heads' outputs are RMS-normed together ("mix.norm"), gated by sigmoid("mix.g" x) and projected by "mix.o".
+     *   TM_MIXER_DELTA: S <- diag(w) S - (a u)(u^T S) + k v^T, o = S^T r, u the unit key, w = exp(-e^(-1/2) sigmoid(w2 tanh(w1 x) + w0)),
+     *     a = sigmoid("mix.a" x + "mix.a.b") per key channel; every head's o is scaled to unit RMS, times "mix.norm", gated like above.
+     *     decay_rank = rows of "mix.w1".  kv_heads = heads, vdim = dim.
+     *   The states are fp32, one per (batch slot, layer run); a sequence whose first row of a forward has position 0 starts from zero.
+     *   TM_MLP_DENSE with act TM_ACT_XIELU ("mlp.act" = [p, q]): z > 0: softplus(p) z^2 + z / 2, else (1/2 + softplus(q)) (e^z - 1 - z) + z / 2.
+     *   TM_MLP_MOE with expert_plain: experts down(relu(up x)^2) ("mlp.e<j>.up|down"); router_softmax: scores soft-max over all experts, the
+     *     `top` largest weight the experts' OUTPUTS times router_scale (not renormalised); shared_ff > 0: an expert of that size
+     *     ("mlp.shared.up|down") runs for every token and is added. */
+    int          post_norm, qkv_bias, qk_norm_w;
+    float        rot_scale;
+    int          window, keep_first;
+    const float* decay; /* TM_MIXER_LIGHTNING: [heads] */
+    int          decay_rank;
+    int          expert_plain, router_softmax;
+    float        router_scale;
+    int          shared_ff;
 } tm_layer_spec;
 typedef struct tm_layered_config {
     int                  width, vocab, n_layers;
@@ -547,6 +571,7 @@ typedef struct tm_layered_config {
     float                norm_eps, norm_offset, residual_mult, logit_scale;
     int                  dtype;
     int                  loop_times; /* 0: no loop tensors */
+    int                  final_layer_norm; /* != 0: the model's last norm is a layer norm with bias ("final.norm", "final.norm.b") */
 } tm_layered_config;
 /* cfg->model is ignored; tp must be 1; quant_policy 0 (the cache holds the activation type) */
 int tm_engine_create_layered(tm_engine** out, const tm_engine_config* cfg, const tm_layered_config* model);
@@ -616,6 +641,8 @@ typedef struct tm_general_attn {
     int             chunk;
     const float*    out_gate;
     int             ld_gate, out_head_stride;
+    /* window > 0: a row at position i sees key j <= i only if i - j < window or j < keep_first */
+    int             window, keep_first;
 } tm_general_attn;
 size_t tm_general_attention_workspace(int rows, int q_heads, int vdim, int splits);
 int    tm_general_attention(const tm_general_attn* a, tm_stream_t st);

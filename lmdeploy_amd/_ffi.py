@@ -73,13 +73,17 @@ class LayerSpec(C.Structure):
                 ('scale', c_float), ('softcap', c_float), ('qtemp_coef', c_float), ('qtemp_every', c_float), ('sink', c_int),
                 ('mlp', c_int), ('ff', c_int), ('act', c_int), ('one_norm', c_int), ('resid_gate', c_int), ('loop_pass', c_int),
                 ('qk_unit_norm', c_int), ('v_unit_norm', c_int), ('dist_bias', c_int), ('out_gate', c_int), ('chunk', c_int),
-                ('kv_rank', c_int), ('rot_dim', c_int), ('rot_base', c_float), ('experts', c_int), ('top', c_int), ('rot_dims', c_int)]
+                ('kv_rank', c_int), ('rot_dim', c_int), ('rot_base', c_float), ('experts', c_int), ('top', c_int), ('rot_dims', c_int),
+                ('post_norm', c_int), ('qkv_bias', c_int), ('qk_norm_w', c_int), ('rot_scale', c_float), ('window', c_int),
+                ('keep_first', c_int), ('decay', POINTER(c_float)), ('decay_rank', c_int), ('expert_plain', c_int),
+                ('router_softmax', c_int), ('router_scale', c_float), ('shared_ff', c_int)]
 
 
 class LayeredConfig(C.Structure):
     """struct tm_layered_config"""
     _fields_ = [('width', c_int), ('vocab', c_int), ('n_layers', c_int), ('layers', POINTER(LayerSpec)), ('norm_eps', c_float),
-                ('norm_offset', c_float), ('residual_mult', c_float), ('logit_scale', c_float), ('dtype', c_int), ('loop_times', c_int)]
+                ('norm_offset', c_float), ('residual_mult', c_float), ('logit_scale', c_float), ('dtype', c_int), ('loop_times', c_int),
+                ('final_layer_norm', c_int)]
 
 
 class StepEntry(C.Structure):
@@ -96,7 +100,7 @@ class GeneralAttn(C.Structure):
                 ('splits', c_int), ('workspace', c_void_p), ('kv', c_void_p), ('ldkv', c_int), ('k_col', c_int), ('v_col', c_int),
                 ('store_kv', c_int), ('kernel', c_int), ('prefill', c_int), ('nseq', c_int), ('max_q_len', c_int), ('cu_q', c_void_p),
                 ('k_len', c_void_p), ('dist_r1', c_void_p), ('dist_r2', c_void_p), ('chunk', c_int), ('out_gate', c_void_p),
-                ('ld_gate', c_int), ('out_head_stride', c_int)]
+                ('ld_gate', c_int), ('out_head_stride', c_int), ('window', c_int), ('keep_first', c_int)]
 
 
 # name -> (restype, argtypes); every int-returning function is a tm_status

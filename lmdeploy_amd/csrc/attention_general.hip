@@ -8,6 +8,8 @@
 //   * chunked visibility:            a row sees the keys of its own chunk of positions only:
 //                                    key >= floor(p / chunk) * chunk, chunks counted from position 0   (chunk = 0: off)
 //   * output gate:                   head h of row t is multiplied by sigmoid(out_gate[t][h])        (out_gate = nullptr: off)
+//   * sliding window:                a row at position p sees key j <= p only if p - j < window or j < keep_first: the window plus
+//                                    the first tokens of the sequence, at their true positions             (window = 0: off)
 // Scores, soft-max weights and the output accumulation are fp32 whatever the cache holds.
 //
 // One launch serves every row of a forward, prefill portions and decoded tokens alike: row t belongs to sequence row_seq[t] at
@@ -98,9 +100,26 @@ __device__ __forceinline__ float ga_dot(const T* __restrict__ k, const float* __
 
 constexpr int kGaMaxDim = 1024;  // key size limit of the row kernel (q in LDS); value size: 64 * VC, VC value channels per lane
 
+// first key of the contiguous range a row sees (its chunk's first position, or the window's)
 __device__ __forceinline__ int ga_first_key(const GeneralAttnParams& p, int pos)
 {
-    return p.chunk > 0 ? pos / p.chunk * p.chunk : 0;
+    const int f = p.chunk > 0 ? pos / p.chunk * p.chunk : 0;
+    return p.window > 0 ? max(f, pos - p.window + 1) : f;
+}
+// keys below that range stay visible while they are among the first ga_keep() positions.  The blocks a row visits are then the
+// `nk` blocks that hold such keys and lie before the range's first block `bf`, followed by bf .. (last block): ga_block_at maps an index of
+// that list to the block; key splits divide the list.
+__device__ __forceinline__ int ga_keep(const GeneralAttnParams& p)
+{
+    return p.window > 0 ? p.keep_first : 0;
+}
+__device__ __forceinline__ int ga_keep_blocks(const GeneralAttnParams& p, int first, int bf, int block_len)
+{
+    return min(bf, (min(ga_keep(p), first) + block_len - 1) / block_len);
+}
+__device__ __forceinline__ int ga_block_at(int bi, int nk, int bf)
+{
+    return bi < nk ? bi : bf + (bi - nk);
 }
 
 // where head h of an output row starts: heads side by side unless the caller spaces them (a batched product reads them at a stride)
@@ -134,9 +153,10 @@ __global__ __launch_bounds__(256) void attn_rows_kernel(GeneralAttnParams p)
     }
     const float qscale = p.scale * ga_query_temp(p, pos);
     const int   nkeys = pos + 1, nblk = (nkeys + p.block_len - 1) / p.block_len;
-    const int   first = ga_first_key(p, pos), bf = first / p.block_len;  // the first visible key and its block
-    const int   per = (nblk - bf + p.splits - 1) / p.splits;
-    const int   b0 = bf + sp * per, b1 = min(nblk, b0 + per);
+    const int   first = ga_first_key(p, pos), bf = first / p.block_len;  // the first key of the visible range and its block
+    const int   keep = ga_keep(p), nk = ga_keep_blocks(p, first, bf, p.block_len), nvis = nk + nblk - bf;
+    const int   per = (nvis + p.splits - 1) / p.splits;
+    const int   i0 = sp * per, i1 = min(nvis, i0 + per);
     const float r1 = p.dist_r1 ? p.dist_r1[h] : 0.f, r2 = p.dist_r1 ? p.dist_r2[h] : 0.f;
     float m = -1e30f, l = 0.f, o[VC];
 #pragma unroll
@@ -147,15 +167,17 @@ __global__ __launch_bounds__(256) void attn_rows_kernel(GeneralAttnParams p)
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    for (int b = b0; b < b1; ++b) {
+    for (int bi = i0; bi < i1; ++bi) {
+        const int   b    = ga_block_at(bi, nk, bf);
         const char* base = (const char*)table[b] + p.layer_offset;
         const T*    kb   = (const T*)base + (size_t)g * p.block_len * D;
         const T*    vb   = (const T*)(base + p.v_offset) + (size_t)g * p.block_len * V;  // [V][block_len]
         const int   n    = min(p.block_len, nkeys - b * p.block_len);
-        const int   jlo  = first - b * p.block_len;  // keys below it lie in an earlier chunk
-        for (int j0 = max(0, jlo) / 64 * 64; j0 < n; j0 += 64) {
+        const int   jlo  = first - b * p.block_len;  // keys below it lie in an earlier chunk / before the window ...
+        const int   klo  = keep - b * p.block_len;   // ... and are seen only as kept first tokens: j < klo
+        for (int j0 = klo > 0 ? 0 : max(0, jlo) / 64 * 64; j0 < n; j0 += 64) {
             const int  j     = j0 + lane;
-            const bool valid = j < n && j >= jlo;
+            const bool valid = j < n && (j >= jlo || j < klo);
             float      sc    = -1e30f;
             if (valid) {
                 sc = ga_modify(p, ga_dot<T>(kb + (size_t)j * D, qs[wave], D), qscale);
@@ -173,7 +195,7 @@ __global__ __launch_bounds__(256) void attn_rows_kernel(GeneralAttnParams p)
                 o[c] *= alpha;
             }
             const int cnt = min(64, n - j0);
-            for (int jj = max(0, jlo - j0); jj < cnt; ++jj) {
+            for (int jj = klo > 0 ? 0 : max(0, jlo - j0); jj < cnt; ++jj) {
                 const float w  = __shfl(pj, jj);
                 const T*    vr = vb + (j0 + jj);
 #pragma unroll
@@ -292,6 +314,7 @@ int launch_general_attention_rows(const GeneralAttnParams& p, hipStream_t st)
     TM_REQUIRE(p.rows >= 0 && p.q_heads >= 1 && p.kv_heads >= 1 && p.q_heads % p.kv_heads == 0, "attention: head counts");
     TM_REQUIRE(p.dim >= 1 && p.dim <= kGaMaxDim && p.vdim >= 1 && p.vdim <= kGaMaxDim, "attention: 1 <= dim, vdim <= 1024");
     TM_REQUIRE(p.chunk >= 0 && (!p.dist_r1 || p.dist_r2) && (!p.out_gate || p.ld_gate >= p.q_heads), "attention: chunk / distance penalty / gate");
+    TM_REQUIRE(p.window >= 0 && p.keep_first >= 0, "attention: window / kept first tokens");
     TM_REQUIRE(p.block_len >= 1 && p.splits >= 1 && (p.splits == 1 || (p.partial_o && p.partial_ml)), "attention: splits / workspace");
     TM_REQUIRE(p.elem_bytes == 2 || p.elem_bytes == 4, "attention: bf16 or fp32");
     TM_REQUIRE(p.qtemp_coef == 0.f || p.qtemp_every > 0.f, "attention: query temperature period");
@@ -339,11 +362,12 @@ __device__ __forceinline__ float ga_tanh_fast(float x)
 // Every key / value fragment is loaded ONCE and serves all RT row tiles; the value fragments are requested before the soft-max
 // arithmetic so that their latency hides under it.  qf: the rows' query fragments; limit: last visible key of the lane's rows
 // (block-relative; < 0: none); kb / vb: the key head's keys [64][D] and transposed values [V][64] of this block.
-// lower: first visible key of the lane's rows (block-relative, may be negative); r1 / r2: the distance penalty of the lane's rows' head
+// lower: first key of the visible range of the lane's rows (block-relative, may be negative); keys below it are seen while < keep_rel
+// (the kept first tokens, block-relative; <= 0: none); r1 / r2: the distance penalty of the lane's rows' head
 // (r1 * log2(1 + r2 * (limit - key)) leaves the score, which lives in the log2 domain; bias = false: none)
 template<int DS, int VT, int RT, bool MASK, bool EAGER>
 __device__ __forceinline__ void ga_block_step(const bf16x8 (&qf)[RT][DS], const __bf16* __restrict__ kb, const __bf16* __restrict__ vb, int D,
-                                              int V, const int (&limit)[RT], const int (&lower)[RT], const float (&qscale)[RT], float cap,
+                                              int V, const int (&limit)[RT], const int (&lower)[RT], int keep_rel, const float (&qscale)[RT], float cap,
                                               float inv_cap, bool bias, float r1, float r2, float (&m)[RT], float (&l)[RT],
                                               floatx4 (&o)[RT][VT])
 {
@@ -415,7 +439,7 @@ __device__ __forceinline__ void ga_block_step(const bf16x8 (&qf)[RT][DS], const 
                     v = fmaf(-r1, __builtin_amdgcn_logf(fmaf(r2, (float)(limit[rt] - key), 1.f)), v);
                 }
                 if (MASK) {
-                    v = (key <= limit[rt] && key >= lower[rt]) ? v : -1e30f;
+                    v = (key <= limit[rt] && (key >= lower[rt] || key < keep_rel)) ? v : -1e30f;
                 }
                 sc[rt][kt][r] = v;
                 bmax          = fmaxf(bmax, v);
@@ -507,7 +531,9 @@ __global__ __launch_bounds__(256) void attn_tiles_kernel(GeneralAttnParams p, in
     const int last_pos = pos0 + min(q_len, row0 + 16 * RT) - 1;  // the wave's last row sees keys 0 .. last_pos
     const int nblk     = last_pos / 64 + 1;
     const int first_lo = ga_first_key(p, pos0 + row0), first_hi = ga_first_key(p, last_pos);  // of the wave's first and last row
-    for (int b = first_lo / 64; b < nblk; ++b) {
+    const int keep = ga_keep(p), bf = first_lo / 64, nk = ga_keep_blocks(p, first_lo, bf, 64);
+    for (int bi = 0; bi < nk + nblk - bf; ++bi) {
+        const int   b    = ga_block_at(bi, nk, bf);
         const char* base = (const char*)table[b] + p.layer_offset;
         int         limit[RT], lower[RT];
 #pragma unroll
@@ -518,10 +544,10 @@ __global__ __launch_bounds__(256) void attn_tiles_kernel(GeneralAttnParams p, in
         const __bf16 *kb = (const __bf16*)base + (size_t)g * 64 * D, *vb = (const __bf16*)(base + p.v_offset) + (size_t)g * 64 * V;
         // every row of the wave sees the whole block (rows beyond the portion are discarded anyway)
         if (b * 64 + 63 <= pos0 + row0 && b * 64 >= first_hi) {
-            ga_block_step<DS, VT, RT, false, false>(qf, kb, vb, D, V, limit, lower, qscale, cap, inv_cap, bias, r1, r2, m, l, o);
+            ga_block_step<DS, VT, RT, false, false>(qf, kb, vb, D, V, limit, lower, 0, qscale, cap, inv_cap, bias, r1, r2, m, l, o);
         }
         else {
-            ga_block_step<DS, VT, RT, true, false>(qf, kb, vb, D, V, limit, lower, qscale, cap, inv_cap, bias, r1, r2, m, l, o);
+            ga_block_step<DS, VT, RT, true, false>(qf, kb, vb, D, V, limit, lower, keep - b * 64, qscale, cap, inv_cap, bias, r1, r2, m, l, o);
         }
     }
 #pragma unroll
@@ -591,13 +617,15 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(GeneralAttnParams p, i
     const bool  bias = p.dist_r1 != nullptr;
     const float r1 = bias ? p.dist_r1[h] : 0.f, r2 = bias ? p.dist_r2[h] : 0.f;  // of the lane's head
     const int first = ga_first_key(p, pos), bf = first / 64;
-    const int nblk = pos / 64 + 1, per = (nblk - bf + p.splits - 1) / p.splits;
-    const int b0 = bf + sp * per, b1 = min(nblk, b0 + per);
-    for (int b = b0 + wave; b < b1; b += 4) {
+    const int keep = ga_keep(p), nk = ga_keep_blocks(p, first, bf, 64);
+    const int nvis = nk + pos / 64 + 1 - bf, per = (nvis + p.splits - 1) / p.splits;
+    const int i0 = sp * per, i1 = min(nvis, i0 + per);
+    for (int bi = i0 + wave; bi < i1; bi += 4) {
+        const int   b    = ga_block_at(bi, nk, bf);
         const char* base = (const char*)table[b] + p.layer_offset;
         const int limit[1] = {pos - b * 64}, lower[1] = {first - b * 64};
         ga_block_step<DS, VT, 1, true, true>(qf, (const __bf16*)base + (size_t)g * 64 * D, (const __bf16*)(base + p.v_offset) + (size_t)g * 64 * V, D,
-                                       V, limit, lower, qscale, cap, inv_cap, bias, r1, r2, m1, l1, o1);
+                                       V, limit, lower, keep - b * 64, qscale, cap, inv_cap, bias, r1, r2, m1, l1, o1);
     }
     const float m = m1[0] * kLn2, l = l1[0];  // back from the log2 domain: the merge below and the split merge kernel use e^x
     floatx4 (&o)[VT] = o1[0];

@@ -709,6 +709,7 @@ int tm_general_attention(const tm_general_attn* a, tm_stream_t st)
     p.nseq = a->nseq, p.max_q_len = a->max_q_len, p.cu_q = a->cu_q, p.k_len = a->k_len;
     p.dist_r1 = a->dist_r1, p.dist_r2 = a->dist_r2, p.chunk = a->chunk, p.out_gate = a->out_gate, p.ld_gate = a->ld_gate;
     p.out_head_stride = a->out_head_stride;
+    p.window = a->window, p.keep_first = a->keep_first;
     if (a->store_kv) {
         TM_REQUIRE(a->kv, "store_kv without kv rows");
         const int rc = launch_kv_store_general(a->kv, a->ldkv, a->k_col, a->v_col, p, (hipStream_t)st);

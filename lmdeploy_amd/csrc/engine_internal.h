@@ -87,6 +87,17 @@ struct LmLayer {
     DenseWeight   wo, gu, down;      // output projection; [gate | up] along N; down (experts: one image per expert in gu / down)
     DenseWeight   uk, uv;            // latent: key expansion transposed [kv_rank][dim] and value expansion [vdim][kv_rank], one image per head
     float *       r1 = nullptr, *r2 = nullptr, *rg1_b = nullptr, *rg2_b = nullptr, *c_norm = nullptr, *inv_freq = nullptr;
+    // post-norm blocks (spec.post_norm): x += LN1(mixer(x)); x += LN2(ff(x)).  `qkv` holds every projection of the mixer's input side by
+    // side (fp32 output), columns
+    //   attention: [q | k | v]   lightning: [q | k | v | gate]   delta rule: [r | k | v | gate | removal rate | decay, inner part]
+    bool               post = false;
+    int                c_end = 0;               // columns of the fused projection
+    int                c_a = 0, c_w1 = 0;       // delta rule: columns of the removal-rate logits and of the decay's inner projection
+    DenseWeight        w2, router, sh_up, sh_down;  // delta: decay outer projection; experts: router, shared expert
+    float *            norm1_b = nullptr, *norm2_b = nullptr, *proj_bias = nullptr, *q_w = nullptr, *k_w = nullptr, *mix_norm = nullptr;
+    float *            w0 = nullptr, *act_par = nullptr, *decay_d = nullptr;
+    std::vector<float> decay_h;                 // lightning: the spec's decays (the spec's pointer is the caller's memory)
+    size_t             state_offset = 0, state_floats = 0;  // this layer run's state inside a slot of the state pool (floats)
 };
 
 struct LayeredModel {
@@ -107,6 +118,14 @@ struct LayeredModel {
     float *              d_proj = nullptr, *d_x0 = nullptr, *d_moe_y = nullptr, *d_topk_w = nullptr;
     void *               d_q = nullptr, *d_plain = nullptr, *d_lat = nullptr, *d_ff = nullptr, *d_xx = nullptr, *d_moe_x = nullptr;
     int *                d_topk_ids = nullptr, *d_offsets = nullptr, *d_f2n = nullptr, *d_en2f = nullptr;
+    // post-norm blocks: a sublayer's fp32 result, state mixers' fp32 output and per-row vectors, the decay's inner activations
+    float *              d_y = nullptr, *d_mixo = nullptr, *d_aux = nullptr, *d_wdec = nullptr, *final_norm_b = nullptr;
+    void*                d_lora = nullptr;
+    int                  ldmix = 0, ldlora = 0;
+    // recurrent states: [max_batch_size + 1 slots][state_slot_floats] fp32; the last slot takes the decode rows of slots without a sequence
+    float*               d_state = nullptr;
+    size_t               state_slot_floats = 0;
+    bool                 has_post = false;
     float*               d_logits_f32 = nullptr;  // [max_logit_rows][vocab]
     int *                d_row_seq = nullptr, *d_row_pos = nullptr, *d_iota = nullptr, *d_want = nullptr, *d_seq_slot = nullptr;
     int *                d_step_ids = nullptr, *d_step_cu_q = nullptr, *d_step_k_len = nullptr;
@@ -127,6 +146,8 @@ struct LmPart {
     const uint64_t* block_ptrs;
     bool            decode;      // one row per sequence
     int             max_q_len;
+    int             slot0  = 0;         // seq_slot == nullptr: sequence i lives in batch slot slot0 + i (the recurrent states are per slot)
+    const int*      active = nullptr;   // [nseq] or nullptr; 0: a placeholder row of a slot without a running sequence
 };
 
 }  // namespace tmk

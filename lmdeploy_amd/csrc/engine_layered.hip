@@ -22,9 +22,28 @@
 //   dense:   a = act(h . gate^T) * (h . up^T)  ONE GEMM over the interleaved [gate | up] image, activation in its epilogue;
 //            x += sigmoid(proj[rg2] + b2) * (a . Wdown^T)
 //   experts: router top-k -> rows sorted by expert, scaled by their score -> the same two products batched over the experts -> gated sum
+//
+// Post-norm blocks (LmLayer::post): the sublayers read the stream itself and a layer norm with bias follows them,
+//   h        = x in the activation type                  (written by the previous block's closing launch)
+//   proj     = h . [every projection of the mixer]^T + bias       ONE GEMM, fp32 output
+//   attention:  launch_attn_prep (weighted per-head norms, rotation) -> paged cache; attention with a window + kept first tokens
+//   lightning / delta rule:  launch_state_mix on the slot's recurrent state (fp32) -> gated group norm
+//   y        = cat . Wo^T (fp32);   x += LN1(y), h = x            one launch
+//   dense:   y = down(xielu(up h));   experts: soft-max router top-k -> rows sorted by expert -> two batched products -> weighted sum
+//            (+ the shared expert);   x += LN2(y), h = x
 #include "engine_internal.h"
 
 namespace tmk {
+
+// out[0] = softplus(p), out[1] = 1/2 + softplus(q): the two numbers of the xIELU activation as the GEMM epilogue reads them
+__global__ void xielu_par_kernel(float* out, const uint16_t* in)
+{
+    if (threadIdx.x < 2) {
+        const float v      = __builtin_bit_cast(float, (uint32_t)in[threadIdx.x] << 16);
+        const float sp     = v > 20.f ? v : log1pf(expf(v));
+        out[threadIdx.x] = threadIdx.x == 0 ? sp : 0.5f + sp;
+    }
+}
 
 __global__ void fill_normal_bf16_kernel(uint16_t* out, size_t n, float mean, float stddev, uint64_t seed)
 {
@@ -166,6 +185,107 @@ static int process_wide_layer(tm_engine* e, int i, LmLayer& L, int dt)
     return 0;
 }
 
+// bf16 vector of a slot -> fp32 at out[0 .. n)
+static int to_f32_at(tm_engine* e, const std::string& name, size_t n, float* out)
+{
+    Slot& s = e->slots[name];
+    TM_REQUIRE(s.filled, "weight not loaded: " + name);
+    bf16_to_f32_kernel<<<(n + 255) / 256, 256, 0, e->stream>>>(out, (const uint16_t*)s.dev, n);
+    TM_HIP_CHECK(hipGetLastError());
+    return 0;
+}
+
+static int process_post_layer(tm_engine* e, int i, LmLayer& L, int dt)
+{
+    const tm_layer_spec& s = L.spec;
+    const int            W = e->lm->cfg.width, H = s.heads, N = L.c_end;
+    TM_TRY(dense_weight_alloc(L.qkv, W, N, dt, e->stream));
+    TM_TRY(place(e, L.qkv, 0, 0, lname(i, s.mixer == TM_MIXER_DELTA ? "mix.r" : "mix.q"), L.n_q, W));
+    TM_TRY(place(e, L.qkv, L.c_k, 0, lname(i, "mix.k"), L.n_k, W));
+    TM_TRY(place(e, L.qkv, L.c_v, 0, lname(i, "mix.v"), L.n_v, W));
+    const bool bias = (s.mixer == TM_MIXER_ATTENTION && s.qkv_bias) || s.mixer == TM_MIXER_DELTA;
+    if (bias) {
+        TM_HIP_CHECK(hipMalloc((void**)&L.proj_bias, (size_t)N * 4));
+        TM_HIP_CHECK(hipMemsetAsync(L.proj_bias, 0, (size_t)N * 4, e->stream));
+    }
+    if (s.mixer == TM_MIXER_ATTENTION) {
+        if (s.qkv_bias) {
+            TM_TRY(to_f32_at(e, lname(i, "mix.q.b"), L.n_q, L.proj_bias));
+            TM_TRY(to_f32_at(e, lname(i, "mix.k.b"), L.n_k, L.proj_bias + L.c_k));
+            TM_TRY(to_f32_at(e, lname(i, "mix.v.b"), L.n_v, L.proj_bias + L.c_v));
+        }
+        if (s.qk_norm_w) {
+            TM_TRY(to_f32(e, lname(i, "mix.q.norm"), s.dim, &L.q_w));
+            TM_TRY(to_f32(e, lname(i, "mix.k.norm"), s.dim, &L.k_w));
+        }
+        if (s.rot_dims > 0) {
+            std::vector<float> f(s.rot_dims / 2);
+            for (int j = 0; j < s.rot_dims / 2; ++j) {
+                f[j] = (float)(std::pow((double)s.rot_base, -2.0 * j / s.rot_dims) / (double)s.rot_scale);
+            }
+            TM_TRY(dmalloc(&L.inv_freq, f.size()));
+            TM_HIP_CHECK(hipMemcpyAsync(L.inv_freq, f.data(), f.size() * 4, hipMemcpyHostToDevice, e->stream));
+            TM_HIP_CHECK(hipStreamSynchronize(e->stream));
+        }
+    }
+    else {
+        TM_TRY(place(e, L.qkv, L.c_g, 0, lname(i, "mix.g"), L.n_att, W));
+        TM_TRY(to_f32(e, lname(i, "mix.norm"), L.n_att, &L.mix_norm));
+        if (s.mixer == TM_MIXER_LIGHTNING) {
+            TM_TRY(dmalloc(&L.decay_d, (size_t)H));
+            TM_HIP_CHECK(hipMemcpyAsync(L.decay_d, L.decay_h.data(), (size_t)H * 4, hipMemcpyHostToDevice, e->stream));
+            TM_HIP_CHECK(hipStreamSynchronize(e->stream));
+        }
+        else {
+            TM_TRY(place(e, L.qkv, L.c_a, 0, lname(i, "mix.a"), L.n_q, W));
+            TM_TRY(place(e, L.qkv, L.c_w1, 0, lname(i, "mix.w1"), s.decay_rank, W));
+            TM_TRY(to_f32_at(e, lname(i, "mix.a.b"), L.n_q, L.proj_bias + L.c_a));
+            TM_TRY(dense_weight_alloc(L.w2, s.decay_rank, L.n_q, dt, e->stream));
+            TM_TRY(place(e, L.w2, 0, 0, lname(i, "mix.w2"), L.n_q, s.decay_rank));
+            TM_TRY(to_f32(e, lname(i, "mix.w0"), L.n_q, &L.w0));
+        }
+    }
+    TM_TRY(dense_weight_alloc(L.wo, L.n_att, W, dt, e->stream));
+    TM_TRY(place(e, L.wo, 0, 0, lname(i, "mix.o"), W, L.n_att));
+    TM_TRY(to_f32(e, lname(i, "norm1"), W, &L.norm1));
+    TM_TRY(to_f32(e, lname(i, "norm1.b"), W, &L.norm1_b));
+    if (s.mlp) {
+        TM_TRY(to_f32(e, lname(i, "norm2"), W, &L.norm2));
+        TM_TRY(to_f32(e, lname(i, "norm2.b"), W, &L.norm2_b));
+    }
+    if (s.mlp == TM_MLP_DENSE) {
+        TM_TRY(dense_weight_alloc(L.up, W, s.ff, dt, e->stream));
+        TM_TRY(place(e, L.up, 0, 0, lname(i, "mlp.up"), s.ff, W));
+        TM_TRY(dense_weight_alloc(L.down, s.ff, W, dt, e->stream));
+        TM_TRY(place(e, L.down, 0, 0, lname(i, "mlp.down"), W, s.ff));
+        if (s.act == TM_ACT_XIELU) {
+            Slot& a = e->slots[lname(i, "mlp.act")];
+            TM_REQUIRE(a.filled, "weight not loaded: " + lname(i, "mlp.act"));
+            TM_TRY(dmalloc(&L.act_par, (size_t)2));
+            xielu_par_kernel<<<1, 64, 0, e->stream>>>(L.act_par, (const uint16_t*)a.dev);
+            TM_HIP_CHECK(hipGetLastError());
+        }
+    }
+    else if (s.mlp == TM_MLP_MOE) {
+        TM_TRY(dense_weight_alloc(L.router, W, s.experts, dt, e->stream));
+        TM_TRY(place(e, L.router, 0, 0, lname(i, "mlp.router"), s.experts, W));
+        TM_TRY(dense_weight_alloc(L.gu, W, s.ff, dt, e->stream, s.experts));
+        TM_TRY(dense_weight_alloc(L.down, s.ff, W, dt, e->stream, s.experts));
+        for (int x = 0; x < s.experts; ++x) {
+            const std::string ex = "mlp.e" + std::to_string(x) + ".";
+            TM_TRY(place(e, L.gu, 0, 0, lname(i, (ex + "up").c_str()), s.ff, W, 0, x));
+            TM_TRY(place(e, L.down, 0, 0, lname(i, (ex + "down").c_str()), W, s.ff, 0, x));
+        }
+        if (s.shared_ff > 0) {
+            TM_TRY(dense_weight_alloc(L.sh_up, W, s.shared_ff, dt, e->stream));
+            TM_TRY(place(e, L.sh_up, 0, 0, lname(i, "mlp.shared.up"), s.shared_ff, W));
+            TM_TRY(dense_weight_alloc(L.sh_down, s.shared_ff, W, dt, e->stream));
+            TM_TRY(place(e, L.sh_down, 0, 0, lname(i, "mlp.shared.down"), W, s.shared_ff));
+        }
+    }
+    return 0;
+}
+
 int layered_process_weights(tm_engine* e)
 {
     LayeredModel&            lm = *e->lm;
@@ -178,6 +298,10 @@ int layered_process_weights(tm_engine* e)
             continue;
         }
         const tm_layer_spec& s = L.spec;
+        if (L.post) {
+            TM_TRY(process_post_layer(e, i, L, dt));
+            continue;
+        }
         if (L.wide) {
             TM_TRY(process_wide_layer(e, i, L, dt));
             continue;
@@ -207,6 +331,9 @@ int layered_process_weights(tm_engine* e)
             L.qkv = S.qkv, L.up = S.up, L.out = S.out, L.norm1 = S.norm1, L.norm2 = S.norm2, L.sink = S.sink;
             L.wo = S.wo, L.gu = S.gu, L.down = S.down, L.uk = S.uk, L.uv = S.uv;
             L.r1 = S.r1, L.r2 = S.r2, L.rg1_b = S.rg1_b, L.rg2_b = S.rg2_b, L.c_norm = S.c_norm, L.inv_freq = S.inv_freq;
+            L.w2 = S.w2, L.router = S.router, L.sh_up = S.sh_up, L.sh_down = S.sh_down, L.norm1_b = S.norm1_b, L.norm2_b = S.norm2_b;
+            L.proj_bias = S.proj_bias, L.q_w = S.q_w, L.k_w = S.k_w, L.mix_norm = S.mix_norm, L.w0 = S.w0, L.act_par = S.act_par;
+            L.decay_d = S.decay_d;
         }
     }
     if (c.loop_times > 0) {
@@ -217,6 +344,9 @@ int layered_process_weights(tm_engine* e)
     TM_TRY(dense_weight_alloc(lm.head, W, c.vocab, dt, e->stream));
     TM_TRY(place(e, lm.head, 0, 0, "head", c.vocab, W));
     TM_TRY(to_f32(e, "final.norm", W, &lm.final_norm));
+    if (c.final_layer_norm) {
+        TM_TRY(to_f32(e, "final.norm.b", W, &lm.final_norm_b));
+    }
     {
         Slot& s = e->slots["embed"];
         TM_REQUIRE(s.filled, "weight not loaded: embed");
@@ -257,11 +387,11 @@ int layered_init_synthetic(tm_engine* e, uint64_t seed)
         const size_t        dot = n.rfind('.');
         const std::string   leaf = dot == std::string::npos ? n : n.substr(dot + 1);
         const bool          isnorm = n.find("norm") != std::string::npos;
-        const bool          vec = isnorm || leaf == "sink" || leaf == "r1" || leaf == "r2" || leaf == "b" || leaf == "step";
+        const bool          vec = isnorm || leaf == "sink" || leaf == "r1" || leaf == "r2" || leaf == "b" || leaf == "step" || leaf == "w0" || leaf == "act";
         // matrices: N(0, 1 / in_features) keeps every projection's output at the scale of its input; vectors: small, around zero (norm
         // weights around 1 - norm_offset; distance-penalty numbers positive)
         float stdv = 0.02f, mean = 0.f;
-        if (isnorm) {
+        if (isnorm && leaf != "b") {
             mean = 1.f - lm.cfg.norm_offset;
         }
         else if (leaf == "r1" || leaf == "r2") {
@@ -315,13 +445,35 @@ int layered_start(tm_engine* e)
     int     max_qkv = 8, max_cat = 32, max_vdim = 0, max_heads = 0;
     int     max_proj = 0, max_q = 0, max_plain = 0, max_lat = 0, max_ff = 0;
     bool    any_moe = false;
+    int     max_mix = 0, max_lora = 0;
     for (LmLayer& L : lm.layers) {
-        L.kv_offset = off;
-        L.v_offset  = (int64_t)L.n_k * c.cache_block_seq_len * lm.elem;
-        off += (int64_t)(L.n_k + L.n_v) * c.cache_block_seq_len * lm.elem;
-        off         = (off + 15) / 16 * 16;
-        max_vdim    = std::max(max_vdim, L.a_vdim);
-        max_heads   = std::max(max_heads, L.spec.heads);
+        const bool stateful = L.spec.mixer == TM_MIXER_LIGHTNING || L.spec.mixer == TM_MIXER_DELTA;
+        if (stateful) {  // a recurrent state per slot instead of cache entries
+            L.state_offset = lm.state_slot_floats;
+            L.state_floats = state_mix_floats(L.spec.heads, L.spec.dim, L.spec.vdim);
+            lm.state_slot_floats += L.state_floats;
+            max_mix  = std::max(max_mix, L.n_att);
+            max_lora = std::max(max_lora, L.w2.Kp);
+        }
+        else {
+            L.kv_offset = off;
+            L.v_offset  = (int64_t)L.n_k * c.cache_block_seq_len * lm.elem;
+            off += (int64_t)(L.n_k + L.n_v) * c.cache_block_seq_len * lm.elem;
+            off         = (off + 15) / 16 * 16;
+            max_vdim    = std::max(max_vdim, L.a_vdim);
+            max_heads   = std::max(max_heads, L.spec.heads);
+        }
+        if (L.post) {
+            max_cat  = std::max(max_cat, L.wo.Kp);
+            max_proj = std::max(max_proj, std::max(L.qkv.N, L.spec.experts));
+            max_q    = std::max(max_q, stateful ? 0 : L.spec.heads * L.a_dim);
+            if (L.spec.mlp) {
+                max_ff     = std::max(max_ff, std::max(L.down.Kp, L.sh_down.Kp));
+                lm.max_top = std::max(lm.max_top, L.spec.mlp == TM_MLP_MOE ? L.spec.top : 1);
+                any_moe    = any_moe || L.spec.mlp == TM_MLP_MOE;
+            }
+            continue;
+        }
         if (!L.wide) {
             max_qkv = std::max(max_qkv, L.qkv.N);
             max_cat = std::max(max_cat, L.out.Kp);
@@ -338,7 +490,8 @@ int layered_start(tm_engine* e)
             any_moe    = any_moe || L.spec.mlp == TM_MLP_MOE;
         }
     }
-    e->block_bytes = off;
+    e->block_bytes = std::max<int64_t>(off, 16);  // (a model without attention layers still has a block pool: the scheduler counts tokens in blocks)
+    max_vdim = std::max(max_vdim, 1), max_heads = std::max(max_heads, 1);
     lm.ldqkv = (max_qkv + 31) / 32 * 32;
     lm.ldcat = max_cat;
     lm.ldv16 = e->vocab_local;
@@ -346,7 +499,7 @@ int layered_start(tm_engine* e)
     if (max_proj > 0) {  // wide blocks
         const size_t TT = T * std::max(1, lm.max_top);  // rows of the experts' products: one per (token, chosen expert)
         lm.ldproj  = (max_proj + 3) / 4 * 4;
-        lm.ldq     = (max_q + 31) / 32 * 32;
+        lm.ldq     = std::max(32, (max_q + 31) / 32 * 32);
         lm.ldplain = std::max(32, max_plain);
         lm.ldlat   = std::max(32, max_lat);
         lm.ldff    = std::max(32, max_ff);
@@ -369,6 +522,18 @@ int layered_start(tm_engine* e)
         lm.ld2w = lm.loop_in.Kp;
         TM_TRY(lm_alloc(&lm.d_x0, T * m.width, st));
         TM_TRY(lm_alloc((char**)&lm.d_xx, T * lm.ld2w * lm.elem, st));
+    }
+    if (lm.has_post) {
+        lm.ldmix  = std::max(4, (max_mix + 3) / 4 * 4);
+        lm.ldlora = std::max(32, max_lora);
+        TM_TRY(lm_alloc(&lm.d_y, T * m.width, st));
+        TM_TRY(lm_alloc(&lm.d_mixo, T * lm.ldmix, st));
+        TM_TRY(lm_alloc(&lm.d_aux, T * lm.ldmix, st));
+        TM_TRY(lm_alloc(&lm.d_wdec, T * lm.ldmix, st));
+        TM_TRY(lm_alloc((char**)&lm.d_lora, T * lm.ldlora * lm.elem, st));
+    }
+    if (lm.state_slot_floats > 0) {
+        TM_TRY(lm_alloc(&lm.d_state, ((size_t)B + 1) * lm.state_slot_floats, st));
     }
     TM_TRY(lm_alloc(&lm.d_res, T * m.width, st));
     TM_TRY(lm_alloc((char**)&lm.d_h1, T * lm.ldw * lm.elem, st));
@@ -447,7 +612,9 @@ void layered_free(tm_engine* e)
         if (L.src == (int)i) {
             dense_weight_free(L.qkv), dense_weight_free(L.up), dense_weight_free(L.out);
             dense_weight_free(L.wo), dense_weight_free(L.gu), dense_weight_free(L.down), dense_weight_free(L.uk), dense_weight_free(L.uv);
-            for (float* p : {L.norm1, L.norm2, L.sink, L.r1, L.r2, L.rg1_b, L.rg2_b, L.c_norm, L.inv_freq}) {
+            dense_weight_free(L.w2), dense_weight_free(L.router), dense_weight_free(L.sh_up), dense_weight_free(L.sh_down);
+            for (float* p : {L.norm1, L.norm2, L.sink, L.r1, L.r2, L.rg1_b, L.rg2_b, L.c_norm, L.inv_freq, L.norm1_b, L.norm2_b, L.proj_bias,
+                             L.q_w, L.k_w, L.mix_norm, L.w0, L.act_par, L.decay_d}) {
                 if (p) {
                     (void)hipFree(p);
                 }
@@ -456,6 +623,11 @@ void layered_free(tm_engine* e)
     }
     dense_weight_free(lm.head);
     dense_weight_free(lm.loop_in);
+    for (void* p : {(void*)lm.d_y, (void*)lm.d_mixo, (void*)lm.d_aux, (void*)lm.d_wdec, lm.d_lora, (void*)lm.d_state, (void*)lm.final_norm_b}) {
+        if (p) {
+            (void)hipFree(p);
+        }
+    }
     for (void* p : {(void*)lm.loop_step, (void*)lm.d_proj, (void*)lm.d_x0, (void*)lm.d_moe_y, (void*)lm.d_topk_w, lm.d_q, lm.d_plain, lm.d_lat,
                     lm.d_ff, lm.d_xx, lm.d_moe_x, (void*)lm.d_topk_ids, (void*)lm.d_offsets, (void*)lm.d_f2n, (void*)lm.d_en2f}) {
         if (p) {
@@ -480,7 +652,7 @@ static GeneralAttnParams attn_params(tm_engine* e, const LmLayer& L, const LmPar
     p.out          = (char*)lm.d_cat + (size_t)P.row0 * lm.ldcat * lm.elem;
     p.ldq          = lm.ldqkv;
     p.ldo          = lm.ldcat;
-    if (L.wide) {
+    if (L.wide || L.post) {
         p.q   = (const char*)lm.d_q + (size_t)P.row0 * lm.ldq * lm.elem;
         p.ldq = lm.ldq;
         if (L.spec.mixer == TM_MIXER_LATENT) {  // the attention output stays in the latent space until the value expansion
@@ -496,6 +668,8 @@ static GeneralAttnParams attn_params(tm_engine* e, const LmLayer& L, const LmPar
     p.dist_r1 = L.r1;
     p.dist_r2 = L.r2;
     p.chunk   = L.spec.chunk;
+    p.window  = L.spec.window;
+    p.keep_first = L.spec.keep_first;
     p.rows         = P.rows;
     p.row_seq      = lm.d_row_seq + P.row0;
     p.row_pos      = lm.d_row_pos + P.row0;
@@ -613,6 +787,106 @@ static int wide_layer(tm_engine* e, const LmLayer& L, int M, const LmPart* parts
     return 0;
 }
 
+// one post-norm block over M rows (see the head of this file); h_ready: lm.d_h1 already holds the stream in the activation type
+static int post_layer(tm_engine* e, const LmLayer& L, int M, const LmPart* parts, int nparts, bool h_ready)
+{
+    LayeredModel&            lm = *e->lm;
+    const tm_layered_config& m  = lm.cfg;
+    const tm_layer_spec&     s  = L.spec;
+    hipStream_t              st = e->stream;
+    const int                W = m.width, H = s.heads;
+    if (!h_ready) {
+        TM_PROF(P_RES_NORM, TM_TRY(launch_act_cast_f32(lm.d_h1, lm.ldw, lm.elem, lm.d_res, W, M, W, 0, st)));
+    }
+    DenseCall pc;
+    pc.epi  = L.proj_bias ? kDenseBiasF32 : kDenseScaleF32;
+    pc.bias = L.proj_bias;
+    TM_PROF(P_GEMM_QKV, TM_TRY(launch_dense_call(L.qkv, lm.d_h1, lm.ldw, lm.d_proj, lm.ldproj, M, pc, st)));
+    if (s.mixer == TM_MIXER_ATTENTION) {
+        AttnPrepExtra ex;
+        ex.q_w = L.q_w, ex.k_w = L.k_w, ex.inv_freq = L.inv_freq, ex.rot_dims = s.rot_dims;
+        for (int i = 0; i < nparts; ++i) {
+            const LmPart&     P = parts[i];
+            GeneralAttnParams p = attn_params(e, L, P);
+            TM_PROF(P_KV_STORE, TM_TRY(launch_attn_prep(lm.d_proj + (size_t)P.row0 * lm.ldproj, lm.ldproj, 0, L.c_k, L.c_v, (void*)p.q, lm.ldq,
+                                                        s.qk_norm_w != 0, false, m.norm_eps, p, st, ex)));
+        }
+        for (int i = 0; i < nparts; ++i) {
+            const LmPart&     P = parts[i];
+            GeneralAttnParams p = attn_params(e, L, P);
+            if (P.decode && lm.decode_splits > 1 && general_attention_workspace_bytes(P.rows, H, L.a_vdim, lm.decode_splits) <= lm.attn_ws_bytes) {
+                p.splits     = lm.decode_splits;
+                p.partial_o  = lm.d_attn_ws;
+                p.partial_ml = lm.d_attn_ws + (size_t)P.rows * H * p.splits * L.a_vdim;
+            }
+            TM_PROF(P_ATTN, TM_TRY(launch_general_attention(p, !P.decode, st)));
+        }
+    }
+    else {
+        const bool delta = s.mixer == TM_MIXER_DELTA;
+        if (delta) {  // decay logits = w2 tanh(w1 h) + w0; then unit keys, removal rates and decays as the recurrence reads them
+            TM_PROF(P_KV_STORE, TM_TRY(launch_act_cast_f32(lm.d_lora, lm.ldlora, lm.elem, lm.d_proj + L.c_w1, lm.ldproj, M, s.decay_rank, 1, st)));
+            DenseCall c;
+            c.epi  = kDenseBiasF32;
+            c.bias = L.w0;
+            TM_PROF(P_GEMM_QKV, TM_TRY(launch_dense_call(L.w2, lm.d_lora, lm.ldlora, lm.d_wdec, lm.ldmix, M, c, st)));
+            TM_PROF(P_KV_STORE, TM_TRY(launch_delta_prep(lm.d_proj, lm.ldproj, L.c_k, L.c_a, lm.d_wdec, lm.ldmix, lm.d_aux, lm.ldmix, M, H, s.dim, st)));
+        }
+        for (int i = 0; i < nparts; ++i) {
+            const LmPart&  P = parts[i];
+            StateMixParams sp;
+            sp.nseq = P.nseq, sp.cu_q = P.cu_q, sp.k_len = P.k_len, sp.seq_slot = P.seq_slot, sp.slot0 = P.slot0, sp.active = P.active;
+            sp.park_slot   = e->cfg.max_batch_size;
+            sp.state       = lm.d_state;
+            sp.slot_stride = lm.state_slot_floats, sp.layer_offset = L.state_offset;
+            sp.heads = H, sp.dim = s.dim, sp.vdim = s.vdim;
+            sp.proj = lm.d_proj + (size_t)P.row0 * lm.ldproj, sp.ld = lm.ldproj;
+            sp.c_q = 0, sp.c_k = L.c_k, sp.c_v = L.c_v, sp.c_a = L.c_a;
+            sp.decay_h = L.decay_d;
+            sp.decay_w = lm.d_wdec + (size_t)P.row0 * lm.ldmix, sp.ld_w = lm.ldmix;
+            sp.unit    = lm.d_aux + (size_t)P.row0 * lm.ldmix, sp.ld_u = lm.ldmix;
+            sp.out     = lm.d_mixo + (size_t)P.row0 * lm.ldmix, sp.ldo = lm.ldmix;
+            TM_PROF(P_ATTN, TM_TRY(launch_state_mix(sp, delta, st)));
+        }
+        TM_PROF(P_ATTN, TM_TRY(launch_gated_group_norm(lm.d_cat, lm.ldcat, lm.elem, lm.d_mixo, lm.ldmix, L.mix_norm, lm.d_proj + L.c_g, lm.ldproj, M,
+                                                       delta ? H : 1, delta ? s.dim : L.n_att, m.norm_eps, st)));
+    }
+    TM_PROF(P_GEMM_O, TM_TRY(launch_dense_linear(L.wo, lm.d_cat, lm.ldcat, lm.d_y, W, M, kDenseScaleF32, 1.f, st)));
+    TM_PROF(P_RES_NORM, TM_TRY(launch_layernorm_add_f32(lm.d_res, lm.d_h1, lm.ldw, lm.elem, lm.d_y, L.norm1, L.norm1_b, m.norm_eps, M, W, st)));
+    if (s.mlp == TM_MLP_NONE) {
+        return 0;
+    }
+    if (s.mlp == TM_MLP_DENSE) {
+        DenseCall c;
+        c.epi     = s.act == TM_ACT_XIELU ? kDenseXielu : kDenseRelu2;
+        c.act_par = L.act_par;
+        TM_PROF(P_GEMM_GATE_UP, TM_TRY(launch_dense_call(L.up, lm.d_h1, lm.ldw, lm.d_ff, lm.ldff, M, c, st)));
+        TM_PROF(P_GEMM_DOWN, TM_TRY(launch_dense_linear(L.down, lm.d_ff, lm.ldff, lm.d_y, W, M, kDenseScaleF32, 1.f, st)));
+    }
+    else {
+        const int k = s.top, E = s.experts;
+        TM_PROF(P_GEMM_GATE_UP, TM_TRY(launch_dense_linear(L.router, lm.d_h1, lm.ldw, lm.d_proj, lm.ldproj, M, kDenseScaleF32, 1.f, st)));
+        TM_PROF(P_GEMM_GATE_UP, TM_TRY(launch_moe_topk_softmax(lm.d_topk_ids, lm.d_topk_w, lm.d_proj, lm.ldproj, M, E, k, s.router_scale, st)));
+        TM_PROF(P_GEMM_GATE_UP, TM_TRY(launch_moe_route(lm.d_offsets, lm.d_f2n, lm.d_en2f, lm.d_topk_ids, M, E, k, st)));
+        TM_PROF(P_GEMM_GATE_UP, TM_TRY(launch_moe_gather(lm.d_moe_x, lm.ldw, lm.d_h1, lm.ldw, lm.elem, lm.d_topk_w, lm.d_en2f, M, W, k, false, st)));
+        DenseCall c;
+        c.epi         = kDenseRelu2;
+        c.count       = E;
+        c.row_offsets = lm.d_offsets;
+        TM_PROF(P_GEMM_GATE_UP, TM_TRY(launch_dense_call(L.gu, lm.d_moe_x, lm.ldw, lm.d_ff, lm.ldff, M * k, c, st)));
+        c.epi = kDenseScaleF32;
+        TM_PROF(P_GEMM_DOWN, TM_TRY(launch_dense_call(L.down, lm.d_ff, lm.ldff, lm.d_moe_y, W, M * k, c, st)));
+        if (s.shared_ff > 0) {  // the shared expert's result opens the sum, the routed experts join it
+            TM_PROF(P_GEMM_GATE_UP, TM_TRY(launch_dense_linear(L.sh_up, lm.d_h1, lm.ldw, lm.d_ff, lm.ldff, M, kDenseRelu2, 1.f, st)));
+            TM_PROF(P_GEMM_DOWN, TM_TRY(launch_dense_linear(L.sh_down, lm.d_ff, lm.ldff, lm.d_y, W, M, kDenseScaleF32, 1.f, st)));
+        }
+        TM_PROF(P_GEMM_DOWN, TM_TRY(launch_moe_combine_f32(lm.d_y, lm.d_moe_y, lm.d_topk_w, lm.d_en2f, nullptr, 0, nullptr, M, W, k, true, st,
+                                                     s.shared_ff <= 0)));
+    }
+    TM_PROF(P_RES_NORM, TM_TRY(launch_layernorm_add_f32(lm.d_res, lm.d_h1, lm.ldw, lm.elem, lm.d_y, L.norm2, L.norm2_b, m.norm_eps, M, W, st)));
+    return 0;
+}
+
 // the layer loop over M rows described by `parts`; leaves the residual stream in lm.d_res
 static int layered_layers(tm_engine* e, const int* d_ids, int M, const LmPart* parts, int nparts)
 {
@@ -638,6 +912,10 @@ static int layered_layers(tm_engine* e, const int* d_ids, int M, const LmPart* p
             c.bias = lm.loop_step + (size_t)s.loop_pass * m.width;
             TM_PROF(P_RES_NORM, TM_TRY(launch_concat2(lm.d_xx, lm.ld2w, lm.elem, lm.d_res, lm.d_x0, M, m.width, st)));
             TM_PROF(P_GEMM_O, TM_TRY(launch_dense_call(lm.loop_in, lm.d_xx, lm.ld2w, lm.d_res, m.width, M, c, st)));
+        }
+        if (L.post) {
+            TM_TRY(post_layer(e, L, M, parts, nparts, li > 0 && lm.layers[li - 1].post));
+            continue;
         }
         if (L.wide) {
             TM_TRY(wide_layer(e, L, M, parts, nparts));
@@ -673,8 +951,14 @@ static int layered_logits(tm_engine* e, const int* rows, int n)
     LayeredModel&            lm = *e->lm;
     const tm_layered_config& m  = lm.cfg;
     TM_REQUIRE(n <= lm.max_logit_rows, "internal: too many logits rows");
-    TM_PROF(P_RES_NORM, TM_TRY(launch_rmsnorm_f32(lm.d_hn, nullptr, lm.ldw, lm.elem, lm.d_res, rows, lm.final_norm, nullptr, m.norm_offset,
-                                                  m.norm_eps, n, m.width, e->stream)));
+    if (m.final_layer_norm) {
+        TM_PROF(P_RES_NORM, TM_TRY(launch_layernorm_f32(lm.d_hn, lm.ldw, lm.elem, lm.d_res, rows, lm.final_norm, lm.final_norm_b, m.norm_eps, n,
+                                                        m.width, e->stream)));
+    }
+    else {
+        TM_PROF(P_RES_NORM, TM_TRY(launch_rmsnorm_f32(lm.d_hn, nullptr, lm.ldw, lm.elem, lm.d_res, rows, lm.final_norm, nullptr, m.norm_offset,
+                                                      m.norm_eps, n, m.width, e->stream)));
+    }
     TM_PROF(P_LM_HEAD, TM_TRY(launch_dense_linear(lm.head, lm.d_hn, lm.ldw, lm.d_logits_f32, m.vocab, n, kDenseScaleF32, m.logit_scale, e->stream)));
     return 0;
 }
@@ -702,9 +986,11 @@ int layered_forward(tm_engine* e, const int* d_ids, int M, int nseq, bool decode
     LmPart parts[2];
     int    np = 0;
     if (md) {  // the decode rows of every batch slot first, on the decode state's own table
-        parts[np++] = LmPart{0, nd, nd, md->cu_q, md->k_len, nullptr, md->block_ptrs, true, 1};
+        parts[np++] = LmPart{0, nd, nd, md->cu_q, md->k_len, nullptr, md->block_ptrs, true, 1, 0, md->active};
     }
-    parts[np++] = LmPart{nd, M - nd, nseq, e->d_cu_q, e->d_k_len, nullptr, e->d_block_ptrs, decode, decode ? 1 : max_q_len};
+    // (the decode step of continuous batching runs every slot: those without a running sequence are placeholders)
+    parts[np++] = LmPart{nd, M - nd, nseq, e->d_cu_q, e->d_k_len, nullptr, e->d_block_ptrs, decode, decode ? 1 : max_q_len, slot0,
+                         decode && e->sched ? e->d_active : nullptr};
     TM_TRY(layered_layers(e, d_ids, M, parts, np));
     if (decode) {
         return layered_head(e, lm.d_iota, nseq, slot0, d_ids, nullptr, M, e->d_k_len, nullptr);
@@ -732,11 +1018,34 @@ int tm_engine_create_layered(tm_engine** out, const tm_engine_config* c, const t
     for (int i = 0; i < m->n_layers; ++i) {
         const tm_layer_spec& s = m->layers[i];
         const std::string at = "layer " + std::to_string(i);
-        TM_REQUIRE(s.mixer == TM_MIXER_ATTENTION || s.mixer == TM_MIXER_LATENT, at + ": unknown mixer");
+        TM_REQUIRE(s.mixer >= TM_MIXER_ATTENTION && s.mixer <= TM_MIXER_DELTA, at + ": unknown mixer");
+        TM_REQUIRE(s.post_norm || (s.mixer != TM_MIXER_LIGHTNING && s.mixer != TM_MIXER_DELTA && !s.qkv_bias && !s.qk_norm_w && s.window == 0
+                                   && !s.expert_plain && !s.router_softmax && s.shared_ff == 0 && s.act != TM_ACT_XIELU),
+                   at + ": state mixers, projection biases, weighted query / key norms, windows, plain experts and xIELU belong to post_norm blocks");
+        TM_REQUIRE(s.window >= 0 && s.keep_first >= 0, at + ": window, keep_first >= 0");
         TM_REQUIRE(s.heads >= 1 && s.kv_heads >= 1 && s.heads % s.kv_heads == 0, at + ": heads % kv_heads");
         TM_REQUIRE(s.dim >= 1 && s.dim <= 256 && s.vdim >= 1 && s.vdim <= 256, at + ": 1 <= dim, vdim <= 256");
         TM_REQUIRE(s.chunk >= 0 && s.loop_pass < m->loop_times, at + ": chunk >= 0, loop_pass < loop_times");
-        if (layer_wide(s)) {
+        if (s.post_norm) {
+            TM_REQUIRE(s.weights_of < 0 && !s.one_norm && !s.resid_gate && s.loop_pass < 0 && !s.sink && !s.dist_bias && !s.out_gate && s.chunk == 0
+                           && !s.qk_unit_norm && !s.v_unit_norm && s.softcap <= 0.f && s.qtemp_coef == 0.f && s.mixer != TM_MIXER_LATENT,
+                       at + ": a post_norm block takes none of the other block forms' switches");
+            TM_REQUIRE(m->final_layer_norm, at + ": post_norm blocks end in a final layer norm");
+            if (s.mixer == TM_MIXER_ATTENTION) {
+                TM_REQUIRE(s.rot_dims >= 0 && s.rot_dims % 2 == 0 && s.rot_dims <= s.dim && s.rot_base > 0.f && s.rot_scale > 0.f,
+                           at + ": rot_dims even and <= dim, rot_base, rot_scale > 0");
+            }
+            else {
+                TM_REQUIRE(s.kv_heads == s.heads, at + ": a state mixer has one key / value head per query head");
+                TM_REQUIRE(s.mixer != TM_MIXER_LIGHTNING || s.decay, at + ": lightning needs one decay per head");
+                TM_REQUIRE(s.mixer != TM_MIXER_DELTA || (s.vdim == s.dim && s.decay_rank >= 1), at + ": delta rule: vdim = dim, decay_rank >= 1");
+            }
+            TM_REQUIRE(s.mlp == TM_MLP_NONE || (s.mlp == TM_MLP_DENSE && s.ff >= 1 && (s.act == TM_ACT_XIELU || s.act == TM_ACT_RELU2))
+                           || (s.mlp == TM_MLP_MOE && s.ff >= 1 && s.expert_plain && s.router_softmax && s.act == TM_ACT_RELU2 && s.experts >= 1
+                               && s.experts <= 1024 && s.top >= 1 && s.top <= s.experts && s.shared_ff >= 0),
+                       at + ": feed-forward of a post_norm block: dense (xIELU | relu^2) or soft-max-routed plain relu^2 experts");
+        }
+        else if (layer_wide(s)) {
             TM_REQUIRE(s.one_norm, at + ": gates, per-head norms, latent attention and gated feed-forwards read ONE norm of the stream (one_norm)");
             TM_REQUIRE(s.mlp == TM_MLP_NONE || ((s.mlp == TM_MLP_GATED || s.mlp == TM_MLP_MOE) && s.ff >= 1 && s.act >= TM_ACT_RELU2 && s.act <= TM_ACT_SILU),
                        at + ": feed-forward");
@@ -792,11 +1101,76 @@ int tm_engine_create_layered(tm_engine** out, const tm_engine_config* c, const t
         L.n_v      = L.spec.kv_heads * L.spec.vdim;
         L.n_att    = L.spec.heads * L.spec.vdim;
         L.a_dim = L.spec.dim, L.a_vdim = L.spec.vdim, L.a_kv = L.spec.kv_heads;
-        L.wide = layer_wide(L.spec);
+        L.post = L.spec.post_norm != 0;
+        L.wide = !L.post && layer_wide(L.spec);
         auto slot = [&](const std::string& name, int64_t rows, int64_t cols) {
             e->slots[name].bytes = rows * cols * 2;
             lm.fan_in[name]      = (int)cols;
         };
+        if (L.post) {
+            const tm_layer_spec& s = L.spec;
+            const int            H = s.heads;
+            lm.has_post = true;
+            L.c_k = L.n_q, L.c_v = L.c_k + L.n_k, L.c_g = L.c_v + L.n_v, L.c_end = L.c_g;
+            slot(lname(i, "norm1"), 1, W);
+            slot(lname(i, "norm1.b"), 1, W);
+            slot(lname(i, s.mixer == TM_MIXER_DELTA ? "mix.r" : "mix.q"), L.n_q, W);
+            slot(lname(i, "mix.k"), L.n_k, W);
+            slot(lname(i, "mix.v"), L.n_v, W);
+            slot(lname(i, "mix.o"), W, L.n_att);
+            if (s.mixer == TM_MIXER_ATTENTION) {
+                if (s.qkv_bias) {
+                    slot(lname(i, "mix.q.b"), 1, L.n_q);
+                    slot(lname(i, "mix.k.b"), 1, L.n_k);
+                    slot(lname(i, "mix.v.b"), 1, L.n_v);
+                }
+                if (s.qk_norm_w) {
+                    slot(lname(i, "mix.q.norm"), 1, s.dim);
+                    slot(lname(i, "mix.k.norm"), 1, s.dim);
+                }
+            }
+            else {
+                L.c_end = L.c_g + L.n_att;
+                slot(lname(i, "mix.g"), L.n_att, W);
+                slot(lname(i, "mix.norm"), 1, L.n_att);
+                if (s.mixer == TM_MIXER_LIGHTNING) {
+                    L.decay_h.assign(s.decay, s.decay + H);
+                    L.spec.decay = nullptr;
+                }
+                else {
+                    L.c_a = L.c_end, L.c_w1 = L.c_a + L.n_q, L.c_end = L.c_w1 + s.decay_rank;
+                    slot(lname(i, "mix.a"), L.n_q, W);
+                    slot(lname(i, "mix.a.b"), 1, L.n_q);
+                    slot(lname(i, "mix.w1"), s.decay_rank, W);
+                    slot(lname(i, "mix.w2"), L.n_q, s.decay_rank);
+                    slot(lname(i, "mix.w0"), 1, L.n_q);
+                }
+            }
+            if (s.mlp) {
+                slot(lname(i, "norm2"), 1, W);
+                slot(lname(i, "norm2.b"), 1, W);
+            }
+            if (s.mlp == TM_MLP_DENSE) {
+                slot(lname(i, "mlp.up"), s.ff, W);
+                slot(lname(i, "mlp.down"), W, s.ff);
+                if (s.act == TM_ACT_XIELU) {
+                    slot(lname(i, "mlp.act"), 1, 2);
+                }
+            }
+            else if (s.mlp == TM_MLP_MOE) {
+                slot(lname(i, "mlp.router"), s.experts, W);
+                for (int x = 0; x < s.experts; ++x) {
+                    const std::string ex = "mlp.e" + std::to_string(x) + ".";
+                    slot(lname(i, (ex + "up").c_str()), s.ff, W);
+                    slot(lname(i, (ex + "down").c_str()), W, s.ff);
+                }
+                if (s.shared_ff > 0) {
+                    slot(lname(i, "mlp.shared.up"), s.shared_ff, W);
+                    slot(lname(i, "mlp.shared.down"), W, s.shared_ff);
+                }
+            }
+            continue;
+        }
         if (L.wide) {
             const tm_layer_spec& s = L.spec;
             const int            H = s.heads;
@@ -889,6 +1263,9 @@ int tm_engine_create_layered(tm_engine** out, const tm_engine_config* c, const t
     }
     e->slots["embed"].bytes      = W * m->vocab * 2;
     e->slots["final.norm"].bytes = W * 2;
+    if (m->final_layer_norm) {
+        e->slots["final.norm.b"].bytes = W * 2;
+    }
     e->slots["head"].bytes       = W * m->vocab * 2;
     *out = e;
     return 0;

@@ -46,6 +46,10 @@ __device__ __forceinline__ void dense_epilogue(void* y, int ldy, int m, int n, f
     else if (c.epi == kDenseBiasF32) {
         ((float*)y)[i] = acc + c.bias[n];
     }
+    else if (c.epi == kDenseXielu) {
+        const float a = c.act_par[0], b = c.act_par[1];
+        ((T*)y)[i]    = (T)(acc > 0.f ? fmaf(a * acc, acc, 0.5f * acc) : fmaf(b, expm1f(acc) - acc, 0.5f * acc));
+    }
     else {  // kDenseResidGate
         const float z = c.gate[(size_t)m * c.ldg + n] + c.gate_bias[n];
         ((float*)y)[i] += acc / (1.f + expf(-z));
@@ -478,7 +482,7 @@ int launch_dense_call(const DenseWeight& d, const void* x, int ldx, void* y, int
     TM_REQUIRE(d.w && x && y && M >= 0 && call.count >= 1 && call.count <= d.count, "dense linear: operands");
     const int n_y = epi == kDenseGatedAct ? call.n_out : d.N;
     TM_REQUIRE(ldx >= d.Kp + (call.count - 1) * call.x_col_stride && ldy >= n_y + (call.count - 1) * call.y_col_stride, "dense linear: row lengths");
-    TM_REQUIRE(epi >= kDenseStore && epi <= kDenseGatedAct, "dense linear: epilogue");
+    TM_REQUIRE(epi >= kDenseStore && epi <= kDenseXielu && (epi != kDenseXielu || call.act_par), "dense linear: epilogue");
     TM_REQUIRE(epi != kDenseGatedAct || (call.n_out >= 1 && dense_pair_rows(call.n_out) <= d.N), "dense linear: paired image");
     TM_REQUIRE(epi != kDenseBiasF32 || call.bias, "dense linear: bias");
     TM_REQUIRE(epi != kDenseResidGate || (call.gate && call.gate_bias && call.ldg >= d.N), "dense linear: gate");

@@ -398,7 +398,7 @@ int launch_kv_store_general(const void* qkv, int ld, int k_col, int v_col, const
 // ([kv_heads][vdim]).  Queries go to q_out [rows][ldq] (head h at h * dim), keys / values into the cache in the general layout.
 template<class T>
 __global__ __launch_bounds__(256) void attn_prep_kernel(const float* __restrict__ proj, int ld, int q_col, int k_col, int v_col, T* __restrict__ q_out,
-                                                        int ldq, int qk_norm, int v_norm, float eps, GeneralAttnParams p)
+                                                        int ldq, int qk_norm, int v_norm, float eps, GeneralAttnParams p, AttnPrepExtra ex)
 {
     const int lane = threadIdx.x & 63, t = blockIdx.x, u = blockIdx.y * 4 + (threadIdx.x >> 6);
     const int H = p.q_heads, G = p.kv_heads;
@@ -416,19 +416,33 @@ __global__ __launch_bounds__(256) void attn_prep_kernel(const float* __restrict_
         }
         inv = 1.0f / sqrtf(group_sum<64>(ss) / (float)n + eps);
     }
+    const int s = p.row_seq[t], pos = p.row_pos[t], ti = pos % p.block_len;
+    // queries and keys: norm weight, then the rotation of the first rd channels (channel i pairs with i + rd / 2), all in fp32
+    const float* nw = kind == 0 ? ex.q_w : (kind == 1 ? ex.k_w : nullptr);
+    const int    rd = kind == 2 ? 0 : ex.rot_dims, half = rd / 2;
+    auto         qk = [&](int i) {
+        const float a = x[i] * inv * (nw ? nw[i] : 1.f);
+        if (i >= rd) {
+            return a;
+        }
+        const int   o = i < half ? i + half : i - half;
+        const float b = x[o] * inv * (nw ? nw[o] : 1.f);
+        float       sn, cs;
+        sincosf((float)pos * ex.inv_freq[i < half ? i : i - half], &sn, &cs);
+        return i < half ? a * cs - b * sn : a * cs + b * sn;
+    };
     if (kind == 0) {
         T* q = q_out + (size_t)t * ldq + (size_t)head * n;
         for (int i = lane; i < n; i += 64) {
-            q[i] = (T)(x[i] * inv);
+            q[i] = (T)qk(i);
         }
         return;
     }
-    const int s = p.row_seq[t], pos = p.row_pos[t], ti = pos % p.block_len;
     char* base = (char*)p.block_ptrs[(size_t)(p.seq_slot ? p.seq_slot[s] : s) * p.block_stride + pos / p.block_len] + p.layer_offset;
     if (kind == 1) {
         T* k = (T*)base + ((size_t)head * p.block_len + ti) * n;
         for (int i = lane; i < n; i += 64) {
-            k[i] = (T)(x[i] * inv);
+            k[i] = (T)qk(i);
         }
     }
     else {
@@ -440,18 +454,19 @@ __global__ __launch_bounds__(256) void attn_prep_kernel(const float* __restrict_
 }
 
 int launch_attn_prep(const float* proj, int ld, int q_col, int k_col, int v_col, void* q_out, int ldq, bool qk_norm, bool v_norm, float eps,
-                     const GeneralAttnParams& p, hipStream_t st)
+                     const GeneralAttnParams& p, hipStream_t st, AttnPrepExtra ex)
 {
     TM_REQUIRE(proj && q_out && p.row_seq && p.row_pos && p.block_ptrs && p.block_stride >= 1, "attn_prep: operands");
+    TM_REQUIRE(ex.rot_dims >= 0 && ex.rot_dims % 2 == 0 && ex.rot_dims <= p.dim && (ex.rot_dims == 0 || ex.inv_freq), "attn_prep: rotation");
     if (p.rows == 0) {
         return 0;
     }
     const dim3 grid(p.rows, (p.q_heads + 2 * p.kv_heads + 3) / 4);
     if (p.elem_bytes == 2) {
-        attn_prep_kernel<__bf16><<<grid, 256, 0, st>>>(proj, ld, q_col, k_col, v_col, (__bf16*)q_out, ldq, qk_norm, v_norm, eps, p);
+        attn_prep_kernel<__bf16><<<grid, 256, 0, st>>>(proj, ld, q_col, k_col, v_col, (__bf16*)q_out, ldq, qk_norm, v_norm, eps, p, ex);
     }
     else {
-        attn_prep_kernel<float><<<grid, 256, 0, st>>>(proj, ld, q_col, k_col, v_col, (float*)q_out, ldq, qk_norm, v_norm, eps, p);
+        attn_prep_kernel<float><<<grid, 256, 0, st>>>(proj, ld, q_col, k_col, v_col, (float*)q_out, ldq, qk_norm, v_norm, eps, p, ex);
     }
     TM_HIP_CHECK(hipGetLastError());
     return 0;

@@ -378,6 +378,52 @@ int launch_moe_topk_sigmoid(int* ids, float* w, const float* logits, int ld, int
     return 0;
 }
 
+// Router scores soft-max(logits) over all experts from fp32 logits; the `k` largest win (ties: the lower index); weight = scale * score.
+__global__ void moe_topk_softmax_kernel(int* __restrict__ ids, float* __restrict__ w, const float* __restrict__ logits, int ld, int T, int E, int k,
+                                        float scale)
+{
+    const int t = blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= T) {
+        return;
+    }
+    const float* z  = logits + (size_t)t * ld;
+    float        mx = z[0];
+    for (int e = 1; e < E; ++e) {
+        mx = fmaxf(mx, z[e]);
+    }
+    float den = 0.f;
+    for (int e = 0; e < E; ++e) {
+        den += expf(z[e] - mx);
+    }
+    for (int j = 0; j < k; ++j) {
+        int   best = -1;
+        float bz   = 0.f;
+        for (int e = 0; e < E; ++e) {
+            bool taken = false;
+            for (int q = 0; q < j; ++q) {
+                taken = taken || ids[(size_t)t * k + q] == e;
+            }
+            if (!taken && (best < 0 || z[e] > bz)) {  // the soft-max is monotonic: order by the logit
+                best = e;
+                bz   = z[e];
+            }
+        }
+        ids[(size_t)t * k + j] = best;
+        w[(size_t)t * k + j]   = scale * (expf(bz - mx) / den);
+    }
+}
+
+int launch_moe_topk_softmax(int* ids, float* w, const float* logits, int ld, int T, int E, int k, float scale, hipStream_t st)
+{
+    TM_REQUIRE(ids && w && logits && E >= 1 && k >= 1 && k <= E && ld >= E, "moe top-k: operands");
+    if (T == 0) {
+        return 0;
+    }
+    moe_topk_softmax_kernel<<<(T + 63) / 64, 64, 0, st>>>(ids, w, logits, ld, T, E, k, scale);
+    TM_HIP_CHECK(hipGetLastError());
+    return 0;
+}
+
 // rows sorted by expert: xs[en2f[j][t]] = (scale ? w[t][j] : 1) * x[t] -- the weight on the expert's INPUT
 template<class T>
 __global__ __launch_bounds__(256) void moe_gather_kernel(T* __restrict__ xs, int lds, const T* __restrict__ x, int ldx, const float* __restrict__ w,
@@ -410,7 +456,8 @@ int launch_moe_gather(void* xs, int lds, const void* x, int ldx, int elem_bytes,
 
 // resid[t] += gate(t) * sum_j (weighted ? w[t][j] : 1) * y[en2f[j][t]], gate(t)[i] = sigmoid(gate[t][i] + gate_bias[i]) (gate == nullptr: 1)
 __global__ void moe_combine_f32_kernel(float* __restrict__ resid, const float* __restrict__ y, const float* __restrict__ w, const int* __restrict__ en2f,
-                                       const float* __restrict__ gate, int ldg, const float* __restrict__ gate_bias, int Tn, int H, int k, int weighted)
+                                       const float* __restrict__ gate, int ldg, const float* __restrict__ gate_bias, int Tn, int H, int k, int weighted,
+                                       int overwrite)
 {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= (size_t)Tn * H) {
@@ -425,18 +472,18 @@ __global__ void moe_combine_f32_kernel(float* __restrict__ resid, const float* _
     if (gate) {
         s = s / (1.f + expf(-(gate[(size_t)t * ldg + c] + gate_bias[c])));
     }
-    resid[i] += s;
+    resid[i] = overwrite ? s : resid[i] + s;
 }
 
 int launch_moe_combine_f32(float* resid, const float* y, const float* w, const int* en2f, const float* gate, int ldg, const float* gate_bias, int T,
-                           int H, int k, bool weighted, hipStream_t st)
+                           int H, int k, bool weighted, hipStream_t st, bool overwrite)
 {
     TM_REQUIRE(resid && y && w && en2f && (!gate || (gate_bias && ldg >= H)), "moe combine: operands");
     const size_t total = (size_t)T * H;
     if (total == 0) {
         return 0;
     }
-    moe_combine_f32_kernel<<<(total + 255) / 256, 256, 0, st>>>(resid, y, w, en2f, gate, ldg, gate_bias, T, H, k, weighted);
+    moe_combine_f32_kernel<<<(total + 255) / 256, 256, 0, st>>>(resid, y, w, en2f, gate, ldg, gate_bias, T, H, k, weighted, overwrite);
     TM_HIP_CHECK(hipGetLastError());
     return 0;
 }

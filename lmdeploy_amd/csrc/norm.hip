@@ -153,4 +153,109 @@ int launch_rmsnorm_f32(void* y0, void* y1, int ldy, int out_elem_bytes, const fl
     return 0;
 }
 
+// layer norm with bias, one workgroup per row; ADD: x[m] += LN(r[m]) and the new row is also written in the activation type
+__device__ __forceinline__ float block_sum_256(float v, float* red)
+{
+    v = group_sum<64>(v);
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) {
+        red[threadIdx.x >> 6] = v;
+    }
+    __syncthreads();
+    return (red[0] + red[1]) + (red[2] + red[3]);
+}
+
+template<class T, bool ADD>
+__global__ __launch_bounds__(256) void layernorm_f32_kernel(T* __restrict__ y, int ldy, float* __restrict__ xs, const float* __restrict__ src,
+                                                            const int* __restrict__ rows, const float* __restrict__ w,
+                                                            const float* __restrict__ b, float eps, int H)
+{
+    __shared__ float red[4];
+    const int    m  = blockIdx.x;
+    const float* r  = src + (size_t)(rows ? rows[m] : m) * H;
+    float        sm = 0.f;
+    for (int i = threadIdx.x; i < H; i += 256) {
+        sm += r[i];
+    }
+    const float mean = block_sum_256(sm, red) / (float)H;
+    float       ss   = 0.f;
+    for (int i = threadIdx.x; i < H; i += 256) {
+        const float d = r[i] - mean;
+        ss            = fmaf(d, d, ss);
+    }
+    const float inv = 1.0f / sqrtf(block_sum_256(ss, red) / (float)H + eps);
+    for (int i = threadIdx.x; i < H; i += 256) {
+        float v = fmaf((r[i] - mean) * inv, w[i], b[i]);
+        if constexpr (ADD) {
+            v += xs[(size_t)m * H + i];
+            xs[(size_t)m * H + i] = v;
+        }
+        y[(size_t)m * ldy + i] = (T)v;
+    }
+}
+
+int launch_layernorm_f32(void* y, int ldy, int out_elem_bytes, const float* x, const int* rows, const float* w, const float* b, float eps, int M,
+                         int H, hipStream_t st)
+{
+    TM_REQUIRE(y && x && w && b && ldy >= H && (out_elem_bytes == 2 || out_elem_bytes == 4), "layernorm_f32: operands");
+    if (M == 0) {
+        return 0;
+    }
+    if (out_elem_bytes == 2) {
+        layernorm_f32_kernel<__bf16, false><<<M, 256, 0, st>>>((__bf16*)y, ldy, nullptr, x, rows, w, b, eps, H);
+    }
+    else {
+        layernorm_f32_kernel<float, false><<<M, 256, 0, st>>>((float*)y, ldy, nullptr, x, rows, w, b, eps, H);
+    }
+    TM_HIP_CHECK(hipGetLastError());
+    return 0;
+}
+
+int launch_layernorm_add_f32(float* x, void* h, int ldh, int h_elem_bytes, const float* r, const float* w, const float* b, float eps, int M, int H,
+                             hipStream_t st)
+{
+    TM_REQUIRE(x && h && r && w && b && ldh >= H && (h_elem_bytes == 2 || h_elem_bytes == 4), "layernorm_add_f32: operands");
+    if (M == 0) {
+        return 0;
+    }
+    if (h_elem_bytes == 2) {
+        layernorm_f32_kernel<__bf16, true><<<M, 256, 0, st>>>((__bf16*)h, ldh, x, r, nullptr, w, b, eps, H);
+    }
+    else {
+        layernorm_f32_kernel<float, true><<<M, 256, 0, st>>>((float*)h, ldh, x, r, nullptr, w, b, eps, H);
+    }
+    TM_HIP_CHECK(hipGetLastError());
+    return 0;
+}
+
+// y = act(x) in the activation type: the stream as a GEMM operand (act 0), tanh of a low-rank projection (act 1)
+template<class T>
+__global__ void act_cast_f32_kernel(T* __restrict__ y, int ldy, const float* __restrict__ x, int ldx, int M, int H, int act)
+{
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (size_t)M * H) {
+        return;
+    }
+    const int   m = (int)(i / H), c = (int)(i % H);
+    const float v = x[(size_t)m * ldx + c];
+    y[(size_t)m * ldy + c] = (T)(act == 1 ? tanhf(v) : v);
+}
+
+int launch_act_cast_f32(void* y, int ldy, int out_elem_bytes, const float* x, int ldx, int M, int H, int act, hipStream_t st)
+{
+    TM_REQUIRE(y && x && ldy >= H && ldx >= H && (out_elem_bytes == 2 || out_elem_bytes == 4), "act_cast_f32: operands");
+    const size_t total = (size_t)M * H;
+    if (total == 0) {
+        return 0;
+    }
+    if (out_elem_bytes == 2) {
+        act_cast_f32_kernel<__bf16><<<(total + 255) / 256, 256, 0, st>>>((__bf16*)y, ldy, x, ldx, M, H, act);
+    }
+    else {
+        act_cast_f32_kernel<float><<<(total + 255) / 256, 256, 0, st>>>((float*)y, ldy, x, ldx, M, H, act);
+    }
+    TM_HIP_CHECK(hipGetLastError());
+    return 0;
+}
+
 }  // namespace tmk

@@ -344,8 +344,9 @@ enum { kDenseBf16 = 0, kDenseF32 = 1 };
 // y_f32 = acc + bias[n] | y_f32 += sigmoid(gate[m][n] + gate_bias[n]) * acc (gated residual sum) |
 // y[m][n] = act(acc_gate[m][n]) * acc_up[m][n] (activation type; the image holds the [gate | up] pair of a gated feed-forward interleaved
 // so that both accumulators of an output element live in one thread: dense_weight_place with half = 1 / 2)
-enum { kDenseStore = 0, kDenseRelu2 = 1, kDenseResidAdd = 2, kDenseScaleF32 = 3, kDenseBiasF32 = 4, kDenseResidGate = 5, kDenseGatedAct = 6 };
-enum { kActRelu2 = 0, kActGeluTanh = 1, kActSilu = 2 };  // (= TM_ACT_*)
+// y = xielu(acc) (activation type; act_par = {softplus(p), 1/2 + softplus(q)}: z > 0: a z^2 + z / 2, else b (e^z - 1 - z) + z / 2)
+enum { kDenseStore = 0, kDenseRelu2 = 1, kDenseResidAdd = 2, kDenseScaleF32 = 3, kDenseBiasF32 = 4, kDenseResidGate = 5, kDenseGatedAct = 6, kDenseXielu = 7 };
+enum { kActRelu2 = 0, kActGeluTanh = 1, kActSilu = 2, kActXielu = 3 };  // (= TM_ACT_*)
 __device__ __forceinline__ float act_apply(int act, float z)
 {
     if (act == kActGeluTanh) {
@@ -382,6 +383,7 @@ struct DenseCall {
     const float* gate  = nullptr;       // kDenseResidGate: gate logits [M][ldg] and their bias [N]
     const float* gate_bias = nullptr;
     int          ldg   = 0;
+    const float* act_par = nullptr;     // kDenseXielu: two fp32 numbers (device)
     int          act = kActRelu2, n_out = 0;  // kDenseGatedAct: the activation and the number of outputs (the image has 2 rows per output)
     int          count = 1;             // items; item g uses image g, x column g * x_col_stride, y column g * y_col_stride ...
     int          x_col_stride = 0, y_col_stride = 0;
@@ -417,6 +419,8 @@ struct GeneralAttnParams {
     const float*    dist_r1 = nullptr;   // [q_heads] or nullptr: score -= r1 * ln(1 + r2 * (position - key position))
     const float*    dist_r2 = nullptr;
     int             chunk = 0;           // > 0: a row sees the keys of its own chunk of positions only (key >= floor(pos / chunk) * chunk)
+    int             window = 0;          // > 0: a row sees key j only if pos - j < window or j < keep_first
+    int             keep_first = 0;
     const float*    out_gate = nullptr;  // [rows][ld_gate] or nullptr: head h of row t is multiplied by sigmoid(out_gate[t][h])
     int             ld_gate = 0;
     int             out_head_stride = 0; // > 0: head h of an output row starts at h * out_head_stride instead of h * vdim
@@ -453,8 +457,14 @@ int launch_rows_prepare(int* row_seq, int* row_pos, const int* cu_q, const int* 
 int launch_kv_store_general(const void* qkv, int ld, int k_col, int v_col, const GeneralAttnParams& layout, hipStream_t st);
 // the same from the fp32 output of a fused projection, with optional unit-RMS scaling per head of queries + keys / of values (no weight);
 // queries -> q_out [rows][ldq] in the cache's element type
+// q_w / k_w (fp32 [dim], may be nullptr): weights of the query / key norm; rot_dims > 0: after the norm the first rot_dims channels of every
+// query and key head turn, channel i with i + rot_dims / 2, by the angle position * inv_freq[i] (fp32)
+struct AttnPrepExtra {
+    const float *q_w = nullptr, *k_w = nullptr, *inv_freq = nullptr;
+    int          rot_dims = 0;
+};
 int launch_attn_prep(const float* proj, int ld, int q_col, int k_col, int v_col, void* q_out, int ldq, bool qk_norm, bool v_norm, float eps,
-                     const GeneralAttnParams& layout, hipStream_t st);
+                     const GeneralAttnParams& layout, hipStream_t st, AttnPrepExtra extra = AttnPrepExtra());
 // latent attention (layout: one key head, dim = C + R, vdim = C): normed latent vector + rotated shared key part -> cache; unrotated query
 // parts -> q_plain (head h at h * plain_stride), rotated query parts -> q_full[h * (C + R) + C ...]
 int launch_latent_prep(const float* proj, int ld, int q_col, int dkv_col, void* q_plain, int ldp, int plain_stride, void* q_full, int ldq,
@@ -464,10 +474,49 @@ int launch_latent_prep(const float* proj, int ld, int q_col, int dkv_col, void* 
 int launch_concat2(void* out, int ldo, int out_elem_bytes, const float* a, const float* b, int M, int H, hipStream_t st);
 // mixture of experts on the fp32 stream: sigmoid router top-k from fp32 logits; gather (optionally scaled) rows in expert order; gated sum
 int launch_moe_topk_sigmoid(int* ids, float* w, const float* logits, int ld, int T, int E, int k, hipStream_t st);
+// soft-max over all E logits; the k largest scores win (ties: the lower index); w = scale * score (not renormalised)
+int launch_moe_topk_softmax(int* ids, float* w, const float* logits, int ld, int T, int E, int k, float scale, hipStream_t st);
 int launch_moe_gather(void* xs, int lds, const void* x, int ldx, int elem_bytes, const float* w, const int* en2f, int T, int H, int k, bool scale,
                       hipStream_t st);
 int launch_moe_combine_f32(float* resid, const float* y, const float* w, const int* en2f, const float* gate, int ldg, const float* gate_bias, int T,
-                           int H, int k, bool weighted, hipStream_t st);
+                           int H, int k, bool weighted, hipStream_t st, bool overwrite = false /* resid = sum instead of resid += sum */);
+// layer norm with bias on the fp32 stream.  launch_layernorm_f32: y[m] = LN(x[rows ? rows[m] : m]) (bf16 | fp32 [M][ldy]);
+// launch_layernorm_add_f32: x[m] += LN(r[m]), and the updated row also goes to h [M][ldh] in the activation type (the next sublayer's
+// GEMM operand).  LN(v) = (v - mean) / sqrt(mean((v - mean)^2) + eps) * w + b, two passes over the row in fp32
+int launch_layernorm_f32(void* y, int ldy, int out_elem_bytes, const float* x, const int* rows, const float* w, const float* b, float eps, int M,
+                         int H, hipStream_t st);
+int launch_layernorm_add_f32(float* x, void* h, int ldh, int h_elem_bytes, const float* r, const float* w, const float* b, float eps, int M, int H,
+                             hipStream_t st);
+// y [M][ldy] (bf16 | fp32) = act(x [M][ldx] fp32), act: 0 none, 1 tanh
+int launch_act_cast_f32(void* y, int ldy, int out_elem_bytes, const float* x, int ldx, int M, int H, int act, hipStream_t st);
+
+// ---- state_mixers.hip: mixers with a recurrent fp32 state per (slot, layer run, head) ---------------------------------------------
+struct StateMixParams {
+    int          nseq = 0;
+    const int*   cu_q = nullptr;      // [nseq + 1] first row of every sequence (rows count from cu_q[0])
+    const int*   k_len = nullptr;     // [nseq] tokens of the sequence including this launch's rows
+    const int*   seq_slot = nullptr;  // [nseq] state slot of a sequence (nullptr: slot0 + s)
+    int          slot0 = 0;
+    const int*   active = nullptr;    // [nseq] or nullptr; 0: the sequence is a placeholder row, its state goes to park_slot
+    int          park_slot = 0;
+    float*       state = nullptr;
+    size_t       slot_stride = 0, layer_offset = 0;  // floats
+    int          heads = 0, dim = 0, vdim = 0;
+    const float* proj = nullptr;      // [rows][ld] fp32: q (delta: r), k, v at the columns below, head by head
+    int          ld = 0, c_q = 0, c_k = 0, c_v = 0, c_a = 0;  // c_a (delta): removal rate times unit key
+    const float* decay_h = nullptr;   // lightning: [heads]
+    const float* decay_w = nullptr;   // delta: [rows][ld_w] decay per key channel
+    const float* unit = nullptr;      // delta: [rows][ld_u] unit keys
+    int          ld_w = 0, ld_u = 0;
+    float*       out = nullptr;       // [rows][ldo] fp32, head h at h * vdim
+    int          ldo = 0;
+};
+size_t state_mix_floats(int heads, int dim, int vdim);  // floats of one layer's state in one slot
+int    launch_state_mix(const StateMixParams& p, bool delta, hipStream_t st);
+int    launch_delta_prep(float* proj, int ld, int c_k, int c_a, float* decay, int ld_w, float* unit, int ld_u, int rows, int heads, int dim,
+                         hipStream_t st);
+int    launch_gated_group_norm(void* y, int ldy, int out_elem_bytes, const float* x, int ldx, const float* w, const float* gate, int ldg, int rows,
+                               int groups, int n, float eps, hipStream_t st);
 // fp32 [n][V] -> fp16 [n][ld] (the sampler's logits rows)
 int launch_f32_to_f16_rows(half_t* out, int ld, const float* in, int n, int V, hipStream_t st);
 

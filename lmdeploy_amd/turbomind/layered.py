@@ -25,9 +25,9 @@ import numpy as np
 from .. import _ffi
 from .engine import Engine
 
-MIXER_ATTENTION, MIXER_LATENT = 1, 2
+MIXER_ATTENTION, MIXER_LATENT, MIXER_LIGHTNING, MIXER_DELTA = 1, 2, 3, 4
 MLP_NONE, MLP_DENSE, MLP_GATED, MLP_MOE = 0, 1, 2, 3
-ACT_RELU2, ACT_GELU_TANH, ACT_SILU = 0, 1, 2
+ACT_RELU2, ACT_GELU_TANH, ACT_SILU, ACT_XIELU = 0, 1, 2, 3
 DTYPES = {'bfloat16': 0, 'bf16': 0, 'float32': 1, 'f32': 1}
 
 
@@ -61,6 +61,18 @@ class LayerSpec:
     experts: int = 0
     top: int = 0
     rot_dims: int = 0             # how many channels of the rotated part turn (0: all of them)
+    post_norm: bool = False       # x += LN(sublayer(x)): the sublayers read the stream, a layer norm with bias follows them
+    qkv_bias: bool = False
+    qk_norm_w: bool = False       # per-head RMS norm of queries and keys with a weight of size dim
+    rot_scale: float = 1.0        # divides every rotation frequency
+    window: int = 0               # > 0: position i sees j only if i - j < window or j < keep_first
+    keep_first: int = 0
+    decay: tuple = ()             # lightning: one decay per head
+    decay_rank: int = 0           # delta rule: inner size of the decay's two-matrix projection
+    expert_plain: bool = False    # experts down(act(up x)) instead of gated ones
+    router_softmax: bool = False  # soft-max scores weight the experts' outputs (times router_scale)
+    router_scale: float = 1.0
+    shared_ff: int = 0            # > 0: an expert of this size runs for every token
 
 
 @dataclass
@@ -76,17 +88,28 @@ class LayeredConfig:
     eos_token_id: int | None = None
     max_position_embeddings: int = 8192
     loop_times: int = 0           # > 0: tensors loop.in / loop.step exist
+    final_layer_norm: bool = False  # the last norm is a layer norm with bias
     names: list = field(default_factory=list)   # tensor prefix of every layer run with tensors of its own ('' -> 'l<index>.')
 
     def native(self, dtype: str):
         """(tm_layered_config, keep-alive array)"""
+        keep = []
+
+        def decays(s):
+            if not s.decay:
+                return None
+            keep.append((C.c_float * len(s.decay))(*s.decay))
+            return keep[-1]
+
         arr = (_ffi.LayerSpec * len(self.layers))(*[
             _ffi.LayerSpec(s.mixer, s.weights_of, s.heads, s.kv_heads, s.dim, s.vdim, s.scale, s.softcap, s.qtemp_coef, s.qtemp_every,
                            int(s.sink), s.mlp, s.ff, s.act, int(s.one_norm), int(s.resid_gate), s.loop_pass, int(s.qk_unit_norm),
-                           int(s.v_unit_norm), int(s.dist_bias), int(s.out_gate), s.chunk, s.kv_rank, s.rot_dim, s.rot_base, s.experts, s.top, s.rot_dims)
+                           int(s.v_unit_norm), int(s.dist_bias), int(s.out_gate), s.chunk, s.kv_rank, s.rot_dim, s.rot_base, s.experts, s.top, s.rot_dims,
+                           int(s.post_norm), int(s.qkv_bias), int(s.qk_norm_w), s.rot_scale, s.window, s.keep_first, decays(s), s.decay_rank,
+                           int(s.expert_plain), int(s.router_softmax), s.router_scale, s.shared_ff)
             for s in self.layers])
         return _ffi.LayeredConfig(self.width, self.vocab, len(self.layers), arr, self.norm_eps, self.norm_offset, self.residual_mult,
-                                  self.logit_scale, DTYPES[dtype], self.loop_times), arr
+                                  self.logit_scale, DTYPES[dtype], self.loop_times, int(self.final_layer_norm)), (arr, keep)
 
     def tensor_name(self, run: int, leaf: str) -> str:
         """checkpoint name of tensor `leaf` of layer run `run` (the engine's slots count layer RUNS; a looped model's file counts layers)"""
@@ -95,6 +118,8 @@ class LayeredConfig:
     def tensor_shapes(self) -> dict:
         """{tensor name: shape} a checkpoint of this config holds"""
         W, out = self.width, {'embed': (self.vocab, self.width), 'final.norm': (self.width,), 'head': (self.vocab, self.width)}
+        if self.final_layer_norm:
+            out['final.norm.b'] = (W,)
         if self.loop_times > 0:
             out['loop.in'], out['loop.step'] = (W, 2 * W), (self.loop_times, W)
         for i, s in enumerate(self.layers):
@@ -102,6 +127,9 @@ class LayeredConfig:
                 continue
             p = f'l{i}.'
             out[p + 'norm1'] = (W,)
+            if s.post_norm:
+                out.update(_post_shapes(p, s, W))
+                continue
             if s.mixer == MIXER_LATENT or s.one_norm:
                 out.update(_wide_shapes(p, s, W))
                 continue
@@ -140,6 +168,90 @@ def _wide_shapes(p: str, s: LayerSpec, W: int) -> dict:
         for e in range(s.experts):
             out[p + f'mlp.e{e}.gate'], out[p + f'mlp.e{e}.up'], out[p + f'mlp.e{e}.down'] = (s.ff, W), (s.ff, W), (W, s.ff)
     return out
+
+
+def _post_shapes(p: str, s: LayerSpec, W: int) -> dict:
+    """tensors of a block whose sublayers read the stream and are followed by a layer norm with bias"""
+    H, d, dv = s.heads, s.dim, s.vdim
+    out = {p + 'norm1.b': (W,), p + 'mix.o': (W, H * dv)}
+    if s.mixer == MIXER_ATTENTION:
+        out[p + 'mix.q'], out[p + 'mix.k'], out[p + 'mix.v'] = (H * d, W), (s.kv_heads * d, W), (s.kv_heads * dv, W)
+        if s.qkv_bias:
+            out[p + 'mix.q.b'], out[p + 'mix.k.b'], out[p + 'mix.v.b'] = (H * d,), (s.kv_heads * d,), (s.kv_heads * dv,)
+        if s.qk_norm_w:
+            out[p + 'mix.q.norm'], out[p + 'mix.k.norm'] = (d,), (d,)
+    elif s.mixer == MIXER_LIGHTNING:
+        out[p + 'mix.q'], out[p + 'mix.k'], out[p + 'mix.v'], out[p + 'mix.g'] = (H * d, W), (H * d, W), (H * dv, W), (H * dv, W)
+        out[p + 'mix.norm'] = (H * dv,)
+    elif s.mixer == MIXER_DELTA:
+        for t in 'rkvga':
+            out[p + 'mix.' + t] = (H * d, W)
+        out[p + 'mix.a.b'], out[p + 'mix.w0'], out[p + 'mix.norm'] = (H * d,), (H * d,), (H * d,)
+        out[p + 'mix.w1'], out[p + 'mix.w2'] = (s.decay_rank, W), (H * d, s.decay_rank)
+    else:
+        raise NotImplementedError(f'{p}: mixer {s.mixer} in a post-norm block')
+    if s.mlp:
+        out[p + 'norm2'], out[p + 'norm2.b'] = (W,), (W,)
+    if s.mlp == MLP_DENSE:
+        out[p + 'mlp.up'], out[p + 'mlp.down'] = (s.ff, W), (W, s.ff)
+        if s.act == ACT_XIELU:
+            out[p + 'mlp.act'] = (2,)
+    elif s.mlp == MLP_MOE:
+        out[p + 'mlp.router'] = (s.experts, W)
+        for e in range(s.experts):
+            out[p + f'mlp.e{e}.up'], out[p + f'mlp.e{e}.down'] = (s.ff, W), (W, s.ff)
+        if s.shared_ff:
+            out[p + 'mlp.shared.up'], out[p + 'mlp.shared.down'] = (s.shared_ff, W), (W, s.shared_ff)
+    return out
+
+
+def _febivik_layer(i: int, L: dict, shapes: dict) -> LayerSpec:
+    m, mlp, kind = L['mixer'], L.get('mlp'), L['type']
+    s = LayerSpec(heads=int(m['heads']), dim=int(m['dim']), post_norm=True)
+    if kind == 'attention':
+        s.mixer, s.kv_heads, s.vdim, s.scale = MIXER_ATTENTION, int(m['kv_heads']), int(m['vdim']), float(m['scale'])
+        s.qkv_bias = s.qk_norm_w = True
+        rot, mask = m.get('rot') or {}, m.get('mask') or {}
+        s.rot_dims, s.rot_base = int(rot.get('dims', 0)), float(rot.get('base', 10000.0))
+        s.rot_scale = float((rot.get('scaling') or {}).get('factor', 1.0))
+        s.window, s.keep_first = int(mask.get('size', 0)), int(mask.get('keep_first', 0))
+        if s.rot_dims % 2 or not 0 <= s.rot_dims <= s.dim or s.rot_scale <= 0:
+            raise ValueError(f'layer {i}: rot.dims must be even and at most dim, the scaling factor positive')
+    elif kind == 'lightning':
+        s.mixer, s.kv_heads, s.vdim = MIXER_LIGHTNING, s.heads, int(m['vdim'])
+        s.decay = tuple(float(v) for v in m['decay'])
+        if len(s.decay) != s.heads:
+            raise ValueError(f'layer {i}: one decay per head')
+    elif kind == 'general_delta':
+        s.mixer, s.kv_heads, s.vdim = MIXER_DELTA, s.heads, s.dim
+        w1 = shapes.get(f'l{i}.mix.w1')     # the inner size of the decay projection is the tensor's own
+        s.decay_rank = int(w1[0]) if w1 else int(m.get('decay_rank', 0) or max(1, min(64, s.dim // 2)))
+    else:
+        raise NotImplementedError(f'layer {i}: mixer {kind!r}')
+    if mlp is None:
+        return s
+    if mlp.get('kind') == 'dense':
+        s.mlp, s.ff, s.act = MLP_DENSE, int(mlp['ff']), ACT_XIELU
+    elif mlp.get('kind') == 'moe':
+        r = mlp['router']
+        s.mlp, s.ff, s.act, s.expert_plain, s.router_softmax = MLP_MOE, int(mlp['expert']['ff']), ACT_RELU2, True, True
+        s.experts, s.top, s.router_scale = int(r['experts']), int(r['top']), float(r.get('scale', 1.0))
+        s.shared_ff = int((mlp.get('shared') or {}).get('ff', 0))
+    else:
+        raise NotImplementedError(f'layer {i}: feed-forward kind {mlp.get("kind")!r}')
+    return s
+
+
+def _febivik(c: dict, shapes: dict | None = None) -> LayeredConfig:
+    """Febivik: blocks x += LN1(mixer(x)); x += LN2(ff(x)) -- the sublayers read the stream itself and a layer norm with bias follows
+    them.  Mixers: lightning (linear attention, one decay per head, a state per head), grouped-query soft-max attention with biases,
+    weighted per-head query / key norms, partial rotation with scaled frequencies and a sliding window that keeps the first tokens, and a
+    generalized delta rule (decay and removal rate per key channel).  Feed-forwards: dense with the xIELU activation, or soft-max-routed
+    squared-ReLU experts plus a shared expert.  `shapes` ({tensor name: shape} of the checkpoint) settles sizes the config leaves to the
+    tensors."""
+    layers = [_febivik_layer(i, L, shapes or {}) for i, L in enumerate(c['layers'])]
+    return LayeredConfig(arch='Febivik', width=int(c['width']), vocab=int(c['vocab']), layers=layers, norm_eps=float(c['norm']['eps']),
+                         norm_offset=0.0, residual_mult=1.0, logit_scale=1.0, eos_token_id=c.get('eos_token_id'), final_layer_norm=True)
 
 
 def _bedenex_layer(i: int, L: dict) -> LayerSpec:
@@ -228,7 +340,8 @@ def _fokonex(c: dict) -> LayeredConfig:
                          logit_scale=float(c['logit_scale']), eos_token_id=c.get('eos_token_id'))
 
 
-FAMILIES = {'Fokonex': _fokonex, 'Bedenex': _bedenex}
+FAMILIES = {'Fokonex': _fokonex, 'Bedenex': _bedenex, 'Febivik': _febivik}
+NEEDS_SHAPES = {'Febivik'}     # readers that take the checkpoint's tensor shapes as a second argument
 
 
 def is_layered(model_path: str) -> bool:
@@ -245,7 +358,18 @@ def read_layered_config(model_path: str) -> LayeredConfig:
     arch = c.get('architecture')
     if arch not in FAMILIES:
         raise NotImplementedError(f'architecture {arch!r}: known layer-list families are {sorted(FAMILIES)}')
+    if arch in NEEDS_SHAPES:
+        st = os.path.join(model_path, 'model.safetensors')
+        return FAMILIES[arch](c, safetensors_shapes(st) if os.path.exists(st) else {})
     return FAMILIES[arch](c)
+
+
+def safetensors_shapes(path: str) -> dict:
+    """{name: shape} from the header of a safetensors file"""
+    with open(path, 'rb') as f:
+        n, = struct.unpack('<Q', f.read(8))
+        header = json.loads(f.read(n).decode('utf-8'))
+    return {k: tuple(v['shape']) for k, v in header.items() if k != '__metadata__'}
 
 
 def read_safetensors(path: str) -> dict:
