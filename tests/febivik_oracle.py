@@ -196,8 +196,8 @@ def forward(cfg, w, tokens, return_layers=False):
 
 
 def router_gap(cfg, w, tokens):
-    """smallest difference between the last chosen and the first rejected router score over all tokens and routed layers: a model
-    whose gap is tiny holds a decision that rounding can turn"""
+    """smallest difference between the router logits of the last chosen and the first rejected expert over all tokens and routed layers: a
+    model whose gap is tiny holds a decision that rounding can turn"""
     eps = float(cfg['norm']['eps'])
     x = w['embed'][np.asarray(tokens)]
     gap = np.inf
@@ -208,11 +208,9 @@ def router_gap(cfg, w, tokens):
         if f is None:
             continue
         if f['kind'] == 'moe' and int(f['router']['top']) < int(f['router']['experts']):
-            z = x @ w[p + 'mlp.router'].T
-            s = np.exp(z - z.max(-1, keepdims=True))
-            s = np.sort(s / s.sum(-1, keepdims=True), -1)[:, ::-1]
+            z = np.sort(x @ w[p + 'mlp.router'].T, -1)[:, ::-1]
             k = int(f['router']['top'])
-            gap = min(gap, float((s[:, k - 1] - s[:, k]).min()))
+            gap = min(gap, float((z[:, k - 1] - z[:, k]).min()))
         y = dense_ff(x, w, p + 'mlp.') if f['kind'] == 'dense' else moe_ff(x, f, w, p + 'mlp.')
         x = x + layer_norm(y, w[p + 'norm2'], w[p + 'norm2.b'], eps)
     return gap
@@ -273,3 +271,75 @@ def random_weights(cfg, seed=0, scale=1.0):
             if f.get('shared'):
                 out[q + 'shared.up'], out[q + 'shared.down'] = mat(f['shared']['ff'], W), mat(W, f['shared']['ff'])
     return out
+
+
+# ---- configurations, checkpoints, generation (test plumbing) ---------------------------------------------------------------------------
+def lightning_layer(heads, dim, vdim, decay, mlp=None):
+    return {'type': 'lightning', 'mixer': {'heads': heads, 'dim': dim, 'vdim': vdim, 'decay': list(decay)}, 'mlp': mlp}
+
+
+def attention_layer(heads, kv_heads, dim, vdim, scale, window=0, keep_first=0, rot_dims=0, base=10000.0, factor=1.0, mlp=None):
+    m = {'heads': heads, 'kv_heads': kv_heads, 'dim': dim, 'vdim': vdim, 'scale': scale}
+    if window:
+        m['mask'] = {'size': window, 'keep_first': keep_first}
+    if rot_dims:
+        m['rot'] = {'dims': rot_dims, 'base': base, 'scaling': {'factor': factor}}
+    return {'type': 'attention', 'mixer': m, 'mlp': mlp}
+
+
+def delta_layer(heads, dim, rank=None, mlp=None):
+    m = {'heads': heads, 'dim': dim}
+    if rank:
+        m['decay_rank'] = rank
+    return {'type': 'general_delta', 'mixer': m, 'mlp': mlp}
+
+
+def dense(ff):
+    return {'kind': 'dense', 'ff': ff}
+
+
+def moe(experts, top, ff, scale=1.0, shared=0):
+    f = {'kind': 'moe', 'expert': {'ff': ff}, 'router': {'experts': experts, 'top': top, 'scale': scale}}
+    if shared:
+        f['shared'] = {'ff': shared}
+    return f
+
+
+def make_config(width, vocab, layers, eps=1e-5):
+    return {'architecture': 'Febivik', 'width': width, 'vocab': vocab, 'norm': {'eps': eps}, 'layers': layers}
+
+
+def bf16_bits(x):
+    b = np.ascontiguousarray(np.asarray(x, np.float32)).view(np.uint32)
+    return ((b + 0x7FFF + ((b >> 16) & 1)) >> 16).astype(np.uint16)
+
+
+def write_checkpoint(folder, cfg, w):
+    """config.json + model.safetensors (8-byte length, JSON header, bf16 data), written by hand"""
+    import json
+    import os
+    import struct
+    os.makedirs(folder, exist_ok=True)
+    with open(os.path.join(folder, 'config.json'), 'w') as f:
+        json.dump(cfg, f)
+    header, blobs, off = {}, [], 0
+    for name in sorted(w):
+        b = bf16_bits(w[name]).astype('<u2').tobytes()
+        header[name] = {'dtype': 'BF16', 'shape': list(np.shape(w[name])), 'data_offsets': [off, off + len(b)]}
+        blobs.append(b)
+        off += len(b)
+    hj = json.dumps(header).encode()
+    with open(os.path.join(folder, 'model.safetensors'), 'wb') as f:
+        f.write(struct.pack('<Q', len(hj)) + hj + b''.join(blobs))
+
+
+def greedy(cfg, w, prompt, n_new):
+    """-> (tokens, margins): arg-max continuation and the top-1 / top-2 logit gap of every step"""
+    toks, out, margins = list(prompt), [], []
+    for _ in range(n_new):
+        lg = forward(cfg, w, toks)[-1]
+        top = np.sort(lg)[-2:]
+        out.append(int(lg.argmax()))
+        margins.append(float(top[1] - top[0]))
+        toks.append(out[-1])
+    return out, margins
