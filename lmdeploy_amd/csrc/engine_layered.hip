@@ -835,6 +835,7 @@ static int post_layer(tm_engine* e, const LmLayer& L, int M, const LmPart* parts
         for (int i = 0; i < nparts; ++i) {
             const LmPart&  P = parts[i];
             StateMixParams sp;
+            sp.max_q_len = P.decode ? 1 : std::max(1, P.max_q_len);
             sp.nseq = P.nseq, sp.cu_q = P.cu_q, sp.k_len = P.k_len, sp.seq_slot = P.seq_slot, sp.slot0 = P.slot0, sp.active = P.active;
             sp.park_slot   = e->cfg.max_batch_size;
             sp.state       = lm.d_state;

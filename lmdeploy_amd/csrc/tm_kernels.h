@@ -492,7 +492,7 @@ int launch_act_cast_f32(void* y, int ldy, int out_elem_bytes, const float* x, in
 
 // ---- state_mixers.hip: mixers with a recurrent fp32 state per (slot, layer run, head) ---------------------------------------------
 struct StateMixParams {
-    int          nseq = 0;
+    int          nseq = 0, max_q_len = 1;  // sequences of the launch; an upper bound of their row counts
     const int*   cu_q = nullptr;      // [nseq + 1] first row of every sequence (rows count from cu_q[0])
     const int*   k_len = nullptr;     // [nseq] tokens of the sequence including this launch's rows
     const int*   seq_slot = nullptr;  // [nseq] state slot of a sequence (nullptr: slot0 + s)

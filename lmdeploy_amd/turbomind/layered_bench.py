@@ -9,6 +9,11 @@ Per kernel category of an eager decode step the table also gives the fraction of
 `bench.py --layered --layered-design bedenex`: the same for Bedenex blocks (chunked attention with unit norms, distance penalty and output
 gate; latent attention; gated residuals; gated-GELU and routed-expert feed-forwards; a looped range of layers) beside the closest
 model the engine serves, the Fokonex blocks above, at equal width, heads, layer count, vocabulary and active feed-forward parameters.
+
+`bench.py --layered --layered-design febivik`: Febivik blocks (lightning and delta-rule state mixers, windowed attention with kept first
+tokens, xIELU and soft-max-routed squared-ReLU experts with a shared expert, layer norms behind the sublayers) beside the closest model
+the engine serves -- the Bedenex blocks above (routed experts, fused fp32 projections) -- at equal width, heads, layer count, vocabulary
+and active feed-forward parameters.
 """
 from __future__ import annotations
 
@@ -84,6 +89,57 @@ def _bedenex_decode_bytes(s, batch, ctx):
     return out
 
 
+FEBIVIK = dict(window=2048, keep_first=4, rot_dims=64, decay_rank=64, experts=8, top=2)
+
+
+def febivik_config(s) -> dict:
+    """config.json of the benchmark model: [lightning + dense, attention + experts, lightning + experts, delta rule + experts] repeated.
+    The dense feed-forward has two matrices of 1.5 x the gated size (equal parameters); experts and the shared expert have a third of
+    it, two experts per token: the active parameters equal the dense block's"""
+    b, H = FEBIVIK, s['heads']
+    ff = s['inter'] * 3 // 2
+    lig = {'heads': H, 'dim': 128, 'vdim': 128, 'decay': [1.0 - 2.0 ** -(5 + 5 * h / max(1, H - 1)) for h in range(H)]}
+    att = {'heads': H, 'kv_heads': s['kv_heads'], 'dim': 128, 'vdim': 128, 'scale': 128 ** -0.5,
+           'mask': {'size': b['window'], 'keep_first': b['keep_first']}, 'rot': {'base': 10000.0, 'dims': b['rot_dims'], 'scaling': {'factor': 4.0}}}
+    dlt = {'heads': H, 'dim': 128, 'decay_rank': b['decay_rank']}
+    dense = {'kind': 'dense', 'ff': ff}
+    moe = {'kind': 'moe', 'expert': {'ff': ff // 3}, 'router': {'experts': b['experts'], 'top': b['top'], 'scale': 1.0}, 'shared': {'ff': ff // 3}}
+    four = [{'type': 'lightning', 'mixer': lig, 'mlp': dense}, {'type': 'attention', 'mixer': att, 'mlp': moe},
+            {'type': 'lightning', 'mixer': lig, 'mlp': moe}, {'type': 'general_delta', 'mixer': dlt, 'mlp': moe}]
+    return {'architecture': 'Febivik', 'width': s['width'], 'vocab': s['vocab'], 'norm': {'eps': 1e-5},
+            'layers': [four[i % 4] for i in range(s['layers'])]}
+
+
+def _febivik_engine(s, batch, session_len, max_prefill):
+    from . import layered
+    cfg = layered.FAMILIES['Febivik'](febivik_config(s))
+    eng = layered.LayeredEngine(cfg, dtype='bfloat16', max_batch_size=batch, session_len=session_len, max_prefill_token_num=max_prefill)
+    eng.init_synthetic(seed=1)
+    eng.start()
+    return eng
+
+
+def _febivik_decode_bytes(s, batch, ctx):
+    """bytes each category of ONE decode step must move: every weight that takes part once (all experts), the cache entries inside the
+    window once per sequence, and every recurrent state read and written once (fp32)"""
+    b, W, H, G, V = FEBIVIK, s['width'], s['heads'], s['kv_heads'], s['vocab']
+    ff = s['inter'] * 3 // 2
+    out = dict(gemm_qkv=0, attention=0, gemm_o=0, gemm_gate_up=0, gemm_down=0, lm_head=2 * W * V)
+    for i in range(s['layers']):
+        kind, moe = ('lightning', 'attention', 'lightning', 'delta')[i % 4], i % 4 != 0
+        if kind == 'attention':
+            out['gemm_qkv'] += 2 * W * (H + 2 * G) * 128
+            out['attention'] += 2 * batch * 2 * G * 128 * min(ctx, b['window'] + b['keep_first'])
+        else:
+            out['gemm_qkv'] += 2 * W * H * 128 * (4 if kind == 'lightning' else 5) + (2 * b['decay_rank'] * (W + H * 128) if kind == 'delta' else 0)
+            out['attention'] += batch * H * 128 * 128 * 4 * 2
+        out['gemm_o'] += 2 * W * H * 128
+        n = (b['experts'] + 1) * (ff // 3) if moe else ff
+        out['gemm_gate_up'] += 2 * W * n + (2 * W * b['experts'] if moe else 0)
+        out['gemm_down'] += 2 * W * n
+    return out
+
+
 def _llama_engine(s, batch, session_len, max_prefill):
     from .engine import Engine
     rope = SimpleNamespace(dim=128, base=10000.0, type='default', factor=1.0, low_freq_factor=1.0, high_freq_factor=4.0,
@@ -143,8 +199,9 @@ def _decode_bytes(s, batch, ctx, fokonex: bool):
 
 def run(steps: int, warmup: int, batch: int, prompt_len: int, sizes=None, design: str = 'fokonex', only_first: bool = False) -> dict:
     res = {}
-    pair = (('fokonex_bf16', _fokonex_engine), ('llama_f16', _llama_engine)) if design == 'fokonex' else \
-        (('bedenex_bf16', _bedenex_engine), ('fokonex_bf16', _fokonex_engine))
+    pair = {'fokonex': (('fokonex_bf16', _fokonex_engine), ('llama_f16', _llama_engine)),
+            'bedenex': (('bedenex_bf16', _bedenex_engine), ('fokonex_bf16', _fokonex_engine)),
+            'febivik': (('febivik_bf16', _febivik_engine), ('bedenex_bf16', _bedenex_engine))}[design]
     if only_first:
         pair = pair[:1]
     for name in (sizes or SIZES):
@@ -156,7 +213,8 @@ def run(steps: int, warmup: int, batch: int, prompt_len: int, sizes=None, design
             eng = make(s, batch, session_len, 8192)
             m = _measure(eng, s['vocab'], batch, prompt_len, steps, warmup, prefill_seqs)
             ctx = prompt_len + warmup + steps // 2
-            need = _bedenex_decode_bytes(s, batch, ctx) if kind == 'bedenex_bf16' else _decode_bytes(s, batch, ctx, kind == 'fokonex_bf16')
+            need = _febivik_decode_bytes(s, batch, ctx) if kind == 'febivik_bf16' else \
+                _bedenex_decode_bytes(s, batch, ctx) if kind == 'bedenex_bf16' else _decode_bytes(s, batch, ctx, kind == 'fokonex_bf16')
             m['decode_hbm_roofline_fraction'] = {k: round(need[k] / HBM_BYTES_PER_S / (m['decode_categories_ms'][k] * 1e-3), 4)
                                                  for k in need if m['decode_categories_ms'].get(k)}
             eng.close()
