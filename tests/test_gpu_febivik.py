@@ -213,7 +213,7 @@ def rel_err(got, ref):
 
 
 ALONE = {
-    'lightning': lambda: fo.make_config(64, 97, [fo.lightning_layer(4, 16, 32, [0.6, 0.9, 0.97, 0.999])]),
+    'lightning': lambda: fo.make_config(64, 97, [fo.lightning_layer(4, 16, 32, [0.55, 0.85, 0.95, 0.9975])]),
     'lightning_one_head_odd_sizes': lambda: fo.make_config(48, 97, [fo.lightning_layer(1, 30, 70, [0.95])]),
     'lightning_large_head': lambda: fo.make_config(64, 97, [fo.lightning_layer(2, 128, 128, [0.99, 0.9])]),
     'attention_window': lambda: fo.make_config(64, 97, [fo.attention_layer(4, 1, 16, 32, 0.5, 33, 2, 8, 500.0, 8.0)]),
