@@ -219,7 +219,8 @@ def _febivik_layer(i: int, L: dict, shapes: dict) -> LayerSpec:
             raise ValueError(f'layer {i}: rot.dims must be even and at most dim, the scaling factor positive')
     elif kind == 'lightning':
         s.mixer, s.kv_heads, s.vdim = MIXER_LIGHTNING, s.heads, int(m['vdim'])
-        s.decay = tuple(float(v) for v in m['decay'])
+        d = m['decay']
+        s.decay = tuple(float(v) for v in d) if isinstance(d, (list, tuple)) else (float(d),) * s.heads
         if len(s.decay) != s.heads:
             raise ValueError(f'layer {i}: one decay per head')
     elif kind == 'general_delta':

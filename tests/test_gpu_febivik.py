@@ -216,6 +216,10 @@ ALONE = {
     'lightning': lambda: fo.make_config(64, 97, [fo.lightning_layer(4, 16, 32, [0.55, 0.85, 0.95, 0.9975])]),
     'lightning_one_head_odd_sizes': lambda: fo.make_config(48, 97, [fo.lightning_layer(1, 30, 70, [0.95])]),
     'lightning_large_head': lambda: fo.make_config(64, 97, [fo.lightning_layer(2, 128, 128, [0.99, 0.9])]),
+    'lightning_head_256': lambda: fo.make_config(48, 97, [fo.lightning_layer(1, 256, 40, [0.98])]),
+    'lightning_head_32': lambda: fo.make_config(48, 97, [fo.lightning_layer(3, 32, 32, [0.7, 0.9, 0.99])]),
+    'delta_head_256': lambda: fo.make_config(48, 97, [fo.delta_layer(1, 256, 6)]),
+    'delta_head_32': lambda: fo.make_config(48, 97, [fo.delta_layer(2, 32, 2)]),
     'attention_window': lambda: fo.make_config(64, 97, [fo.attention_layer(4, 1, 16, 32, 0.5, 33, 2, 8, 500.0, 8.0)]),
     'attention_plain_causal_full_rotation': lambda: fo.make_config(48, 97, [fo.attention_layer(2, 2, 40, 8, 0.2, 0, 0, 40)]),
     'attention_no_rotation_window_1': lambda: fo.make_config(48, 97, [fo.attention_layer(2, 1, 24, 24, 0.2, 1, 1)]),
