@@ -91,6 +91,7 @@ struct LmLayer {
     // side (fp32 output), columns
     //   attention: [q | k | v]   lightning: [q | k | v | gate]   delta rule: [r | k | v | gate | removal rate | decay, inner part]
     bool               post = false;
+    bool               shared_fused = false;    // the shared expert is one more item of the experts' batched products (shared_ff <= ff)
     int                c_end = 0;               // columns of the fused projection
     int                c_a = 0, c_w1 = 0;       // delta rule: columns of the removal-rate logits and of the decay's inner projection
     DenseWeight        w2, router, sh_up, sh_down;  // delta: decay outer projection; experts: router, shared expert

@@ -269,14 +269,20 @@ static int process_post_layer(tm_engine* e, int i, LmLayer& L, int dt)
     else if (s.mlp == TM_MLP_MOE) {
         TM_TRY(dense_weight_alloc(L.router, W, s.experts, dt, e->stream));
         TM_TRY(place(e, L.router, 0, 0, lname(i, "mlp.router"), s.experts, W));
-        TM_TRY(dense_weight_alloc(L.gu, W, s.ff, dt, e->stream, s.experts));
-        TM_TRY(dense_weight_alloc(L.down, s.ff, W, dt, e->stream, s.experts));
+        // a shared expert no larger than the routed ones is one more image of their batched products (zero-padded to their size)
+        const int items = s.experts + (L.shared_fused ? 1 : 0);
+        TM_TRY(dense_weight_alloc(L.gu, W, s.ff, dt, e->stream, items));
+        TM_TRY(dense_weight_alloc(L.down, s.ff, W, dt, e->stream, items));
         for (int x = 0; x < s.experts; ++x) {
             const std::string ex = "mlp.e" + std::to_string(x) + ".";
             TM_TRY(place(e, L.gu, 0, 0, lname(i, (ex + "up").c_str()), s.ff, W, 0, x));
             TM_TRY(place(e, L.down, 0, 0, lname(i, (ex + "down").c_str()), W, s.ff, 0, x));
         }
-        if (s.shared_ff > 0) {
+        if (L.shared_fused) {
+            TM_TRY(place(e, L.gu, 0, 0, lname(i, "mlp.shared.up"), s.shared_ff, W, 0, s.experts));
+            TM_TRY(place(e, L.down, 0, 0, lname(i, "mlp.shared.down"), W, s.shared_ff, 0, s.experts));
+        }
+        else if (s.shared_ff > 0) {
             TM_TRY(dense_weight_alloc(L.sh_up, W, s.shared_ff, dt, e->stream));
             TM_TRY(place(e, L.sh_up, 0, 0, lname(i, "mlp.shared.up"), s.shared_ff, W));
             TM_TRY(dense_weight_alloc(L.sh_down, s.shared_ff, W, dt, e->stream));
@@ -469,7 +475,7 @@ int layered_start(tm_engine* e)
             max_q    = std::max(max_q, stateful ? 0 : L.spec.heads * L.a_dim);
             if (L.spec.mlp) {
                 max_ff     = std::max(max_ff, std::max(L.down.Kp, L.sh_down.Kp));
-                lm.max_top = std::max(lm.max_top, L.spec.mlp == TM_MLP_MOE ? L.spec.top : 1);
+                lm.max_top = std::max(lm.max_top, L.spec.mlp == TM_MLP_MOE ? L.spec.top + (L.shared_fused ? 1 : 0) : 1);
                 any_moe    = any_moe || L.spec.mlp == TM_MLP_MOE;
             }
             continue;
@@ -870,19 +876,31 @@ static int post_layer(tm_engine* e, const LmLayer& L, int M, const LmPart* parts
         TM_PROF(P_GEMM_GATE_UP, TM_TRY(launch_moe_topk_softmax(lm.d_topk_ids, lm.d_topk_w, lm.d_proj, lm.ldproj, M, E, k, s.router_scale, st)));
         TM_PROF(P_GEMM_GATE_UP, TM_TRY(launch_moe_route(lm.d_offsets, lm.d_f2n, lm.d_en2f, lm.d_topk_ids, M, E, k, st)));
         TM_PROF(P_GEMM_GATE_UP, TM_TRY(launch_moe_gather(lm.d_moe_x, lm.ldw, lm.d_h1, lm.ldw, lm.elem, lm.d_topk_w, lm.d_en2f, M, W, k, false, st)));
+        int rows = M * k;
+        if (L.shared_fused) {  // the shared expert: item E of the batched products over a copy of all rows behind the routed ones
+            TM_HIP_CHECK(hipMemcpyAsync((char*)lm.d_moe_x + (size_t)rows * lm.ldw * lm.elem, lm.d_h1, (size_t)M * lm.ldw * lm.elem, hipMemcpyDeviceToDevice, st));
+            TM_PROF(P_GEMM_GATE_UP, TM_TRY(launch_moe_extend_offsets(lm.d_offsets, E, M, st)));
+            rows += M;
+        }
         DenseCall c;
         c.epi         = kDenseRelu2;
-        c.count       = E;
+        c.count       = E + (L.shared_fused ? 1 : 0);
         c.row_offsets = lm.d_offsets;
-        TM_PROF(P_GEMM_GATE_UP, TM_TRY(launch_dense_call(L.gu, lm.d_moe_x, lm.ldw, lm.d_ff, lm.ldff, M * k, c, st)));
+        TM_PROF(P_GEMM_GATE_UP, TM_TRY(launch_dense_call(L.gu, lm.d_moe_x, lm.ldw, lm.d_ff, lm.ldff, rows, c, st)));
         c.epi = kDenseScaleF32;
-        TM_PROF(P_GEMM_DOWN, TM_TRY(launch_dense_call(L.down, lm.d_ff, lm.ldff, lm.d_moe_y, W, M * k, c, st)));
-        if (s.shared_ff > 0) {  // the shared expert's result opens the sum, the routed experts join it
+        TM_PROF(P_GEMM_DOWN, TM_TRY(launch_dense_call(L.down, lm.d_ff, lm.ldff, lm.d_moe_y, W, rows, c, st)));
+        if (L.shared_fused) {
+            TM_PROF(P_GEMM_DOWN, TM_TRY(launch_moe_combine_f32(lm.d_y, lm.d_moe_y, lm.d_topk_w, lm.d_en2f, nullptr, 0, nullptr, M, W, k, true, st, true,
+                                                         lm.d_moe_y + (size_t)M * k * W)));
+        }
+        else if (s.shared_ff > 0) {  // the shared expert's result opens the sum, the routed experts join it
             TM_PROF(P_GEMM_GATE_UP, TM_TRY(launch_dense_linear(L.sh_up, lm.d_h1, lm.ldw, lm.d_ff, lm.ldff, M, kDenseRelu2, 1.f, st)));
             TM_PROF(P_GEMM_DOWN, TM_TRY(launch_dense_linear(L.sh_down, lm.d_ff, lm.ldff, lm.d_y, W, M, kDenseScaleF32, 1.f, st)));
         }
-        TM_PROF(P_GEMM_DOWN, TM_TRY(launch_moe_combine_f32(lm.d_y, lm.d_moe_y, lm.d_topk_w, lm.d_en2f, nullptr, 0, nullptr, M, W, k, true, st,
-                                                     s.shared_ff <= 0)));
+        if (!L.shared_fused) {
+            TM_PROF(P_GEMM_DOWN, TM_TRY(launch_moe_combine_f32(lm.d_y, lm.d_moe_y, lm.d_topk_w, lm.d_en2f, nullptr, 0, nullptr, M, W, k, true, st,
+                                                         s.shared_ff <= 0)));
+        }
     }
     TM_PROF(P_RES_NORM, TM_TRY(launch_layernorm_add_f32(lm.d_res, lm.d_h1, lm.ldw, lm.elem, lm.d_y, L.norm2, L.norm2_b, m.norm_eps, M, W, st)));
     return 0;
@@ -1113,6 +1131,7 @@ int tm_engine_create_layered(tm_engine** out, const tm_engine_config* c, const t
             const int            H = s.heads;
             lm.has_post = true;
             L.c_k = L.n_q, L.c_v = L.c_k + L.n_k, L.c_g = L.c_v + L.n_v, L.c_end = L.c_g;
+            L.shared_fused = s.mlp == TM_MLP_MOE && s.shared_ff > 0 && s.shared_ff <= s.ff;
             slot(lname(i, "norm1"), 1, W);
             slot(lname(i, "norm1.b"), 1, W);
             slot(lname(i, s.mixer == TM_MIXER_DELTA ? "mix.r" : "mix.q"), L.n_q, W);

@@ -457,7 +457,7 @@ int launch_moe_gather(void* xs, int lds, const void* x, int ldx, int elem_bytes,
 // resid[t] += gate(t) * sum_j (weighted ? w[t][j] : 1) * y[en2f[j][t]], gate(t)[i] = sigmoid(gate[t][i] + gate_bias[i]) (gate == nullptr: 1)
 __global__ void moe_combine_f32_kernel(float* __restrict__ resid, const float* __restrict__ y, const float* __restrict__ w, const int* __restrict__ en2f,
                                        const float* __restrict__ gate, int ldg, const float* __restrict__ gate_bias, int Tn, int H, int k, int weighted,
-                                       int overwrite)
+                                       int overwrite, const float* __restrict__ add)
 {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= (size_t)Tn * H) {
@@ -472,18 +472,31 @@ __global__ void moe_combine_f32_kernel(float* __restrict__ resid, const float* _
     if (gate) {
         s = s / (1.f + expf(-(gate[(size_t)t * ldg + c] + gate_bias[c])));
     }
-    resid[i] = overwrite ? s : resid[i] + s;
+    resid[i] = overwrite ? (add ? add[i] + s : s) : resid[i] + s;
 }
 
 int launch_moe_combine_f32(float* resid, const float* y, const float* w, const int* en2f, const float* gate, int ldg, const float* gate_bias, int T,
-                           int H, int k, bool weighted, hipStream_t st, bool overwrite)
+                           int H, int k, bool weighted, hipStream_t st, bool overwrite, const float* add)
 {
     TM_REQUIRE(resid && y && w && en2f && (!gate || (gate_bias && ldg >= H)), "moe combine: operands");
     const size_t total = (size_t)T * H;
     if (total == 0) {
         return 0;
     }
-    moe_combine_f32_kernel<<<(total + 255) / 256, 256, 0, st>>>(resid, y, w, en2f, gate, ldg, gate_bias, T, H, k, weighted, overwrite);
+    moe_combine_f32_kernel<<<(total + 255) / 256, 256, 0, st>>>(resid, y, w, en2f, gate, ldg, gate_bias, T, H, k, weighted, overwrite, add);
+    TM_HIP_CHECK(hipGetLastError());
+    return 0;
+}
+
+__global__ void moe_extend_offsets_kernel(int* offsets, int n, int extra)
+{
+    offsets[n + 1] = offsets[n] + extra;
+}
+
+int launch_moe_extend_offsets(int* offsets, int n, int extra, hipStream_t st)
+{
+    TM_REQUIRE(offsets && n >= 0 && extra >= 0, "moe offsets: operands");
+    moe_extend_offsets_kernel<<<1, 1, 0, st>>>(offsets, n, extra);
     TM_HIP_CHECK(hipGetLastError());
     return 0;
 }

@@ -194,6 +194,62 @@ __global__ __launch_bounds__(256) void layernorm_f32_kernel(T* __restrict__ y, i
     }
 }
 
+// the same with the row held in registers (H <= 256 * NR): one pass over memory instead of three
+template<class T, bool ADD, int NR>
+__global__ __launch_bounds__(256) void layernorm_f32_reg_kernel(T* __restrict__ y, int ldy, float* __restrict__ xs, const float* __restrict__ src,
+                                                                const int* __restrict__ rows, const float* __restrict__ w,
+                                                                const float* __restrict__ b, float eps, int H)
+{
+    __shared__ float red[4];
+    const int    m = blockIdx.x;
+    const float* r = src + (size_t)(rows ? rows[m] : m) * H;
+    float        v[NR], sm = 0.f;
+#pragma unroll
+    for (int q = 0; q < NR; ++q) {
+        const int i = threadIdx.x + q * 256;
+        v[q]        = i < H ? r[i] : 0.f;
+        sm += v[q];
+    }
+    const float mean = block_sum_256(sm, red) / (float)H;
+    float       ss   = 0.f;
+#pragma unroll
+    for (int q = 0; q < NR; ++q) {
+        const float d = threadIdx.x + q * 256 < H ? v[q] - mean : 0.f;
+        ss            = fmaf(d, d, ss);
+    }
+    const float inv = 1.0f / sqrtf(block_sum_256(ss, red) / (float)H + eps);
+#pragma unroll
+    for (int q = 0; q < NR; ++q) {
+        const int i = threadIdx.x + q * 256;
+        if (i < H) {
+            float o = fmaf((v[q] - mean) * inv, w[i], b[i]);
+            if constexpr (ADD) {
+                o += xs[(size_t)m * H + i];
+                xs[(size_t)m * H + i] = o;
+            }
+            y[(size_t)m * ldy + i] = (T)o;
+        }
+    }
+}
+
+template<class T, bool ADD>
+static void launch_layernorm_any(T* y, int ldy, float* xs, const float* src, const int* rows, const float* w, const float* b, float eps, int M, int H,
+                                 hipStream_t st)
+{
+    if (H <= 1024) {
+        layernorm_f32_reg_kernel<T, ADD, 4><<<M, 256, 0, st>>>(y, ldy, xs, src, rows, w, b, eps, H);
+    }
+    else if (H <= 4096) {
+        layernorm_f32_reg_kernel<T, ADD, 16><<<M, 256, 0, st>>>(y, ldy, xs, src, rows, w, b, eps, H);
+    }
+    else if (H <= 8192) {
+        layernorm_f32_reg_kernel<T, ADD, 32><<<M, 256, 0, st>>>(y, ldy, xs, src, rows, w, b, eps, H);
+    }
+    else {
+        layernorm_f32_kernel<T, ADD><<<M, 256, 0, st>>>(y, ldy, xs, src, rows, w, b, eps, H);
+    }
+}
+
 int launch_layernorm_f32(void* y, int ldy, int out_elem_bytes, const float* x, const int* rows, const float* w, const float* b, float eps, int M,
                          int H, hipStream_t st)
 {
@@ -202,10 +258,10 @@ int launch_layernorm_f32(void* y, int ldy, int out_elem_bytes, const float* x, c
         return 0;
     }
     if (out_elem_bytes == 2) {
-        layernorm_f32_kernel<__bf16, false><<<M, 256, 0, st>>>((__bf16*)y, ldy, nullptr, x, rows, w, b, eps, H);
+        launch_layernorm_any<__bf16, false>((__bf16*)y, ldy, nullptr, x, rows, w, b, eps, M, H, st);
     }
     else {
-        layernorm_f32_kernel<float, false><<<M, 256, 0, st>>>((float*)y, ldy, nullptr, x, rows, w, b, eps, H);
+        launch_layernorm_any<float, false>((float*)y, ldy, nullptr, x, rows, w, b, eps, M, H, st);
     }
     TM_HIP_CHECK(hipGetLastError());
     return 0;
@@ -219,10 +275,10 @@ int launch_layernorm_add_f32(float* x, void* h, int ldh, int h_elem_bytes, const
         return 0;
     }
     if (h_elem_bytes == 2) {
-        layernorm_f32_kernel<__bf16, true><<<M, 256, 0, st>>>((__bf16*)h, ldh, x, r, nullptr, w, b, eps, H);
+        launch_layernorm_any<__bf16, true>((__bf16*)h, ldh, x, r, nullptr, w, b, eps, M, H, st);
     }
     else {
-        layernorm_f32_kernel<float, true><<<M, 256, 0, st>>>((float*)h, ldh, x, r, nullptr, w, b, eps, H);
+        launch_layernorm_any<float, true>((float*)h, ldh, x, r, nullptr, w, b, eps, M, H, st);
     }
     TM_HIP_CHECK(hipGetLastError());
     return 0;

@@ -479,7 +479,10 @@ int launch_moe_topk_softmax(int* ids, float* w, const float* logits, int ld, int
 int launch_moe_gather(void* xs, int lds, const void* x, int ldx, int elem_bytes, const float* w, const int* en2f, int T, int H, int k, bool scale,
                       hipStream_t st);
 int launch_moe_combine_f32(float* resid, const float* y, const float* w, const int* en2f, const float* gate, int ldg, const float* gate_bias, int T,
-                           int H, int k, bool weighted, hipStream_t st, bool overwrite = false /* resid = sum instead of resid += sum */);
+                           int H, int k, bool weighted, hipStream_t st, bool overwrite = false /* resid = sum instead of resid += sum */,
+                           const float* add = nullptr /* overwrite: resid = add + sum ([T][H]) */);
+// offsets[n + 1] = offsets[n] + extra: one more item behind the n items of a routing table (rows that every token sends)
+int launch_moe_extend_offsets(int* offsets, int n, int extra, hipStream_t st);
 // layer norm with bias on the fp32 stream.  launch_layernorm_f32: y[m] = LN(x[rows ? rows[m] : m]) (bf16 | fp32 [M][ldy]);
 // launch_layernorm_add_f32: x[m] += LN(r[m]), and the updated row also goes to h [M][ldh] in the activation type (the next sublayer's
 // GEMM operand).  LN(v) = (v - mean) / sqrt(mean((v - mean)^2) + eps) * w + b, two passes over the row in fp32
