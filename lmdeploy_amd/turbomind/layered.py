@@ -209,16 +209,17 @@ def _febivik_layer(i: int, L: dict, shapes: dict) -> LayerSpec:
     m, mlp, kind = L['mixer'], L.get('mlp'), L['type']
     s = LayerSpec(heads=int(m['heads']), dim=int(m['dim']), post_norm=True)
     if kind == 'attention':
-        s.mixer, s.kv_heads, s.vdim, s.scale = MIXER_ATTENTION, int(m['kv_heads']), int(m['vdim']), float(m['scale'])
+        s.mixer, s.kv_heads, s.vdim = MIXER_ATTENTION, int(m.get('kv_heads', s.heads)), int(m.get('vdim', s.dim))
+        s.scale = float(m['scale']) if 'scale' in m else s.dim ** -0.5
         s.qkv_bias = s.qk_norm_w = True
         rot, mask = m.get('rot') or {}, m.get('mask') or {}
-        s.rot_dims, s.rot_base = int(rot.get('dims', 0)), float(rot.get('base', 10000.0))
+        s.rot_dims, s.rot_base = int(rot.get('dims', s.dim)) if rot else 0, float(rot.get('base', 10000.0))      # (a rotation without 'dims' turns the whole head)
         s.rot_scale = float((rot.get('scaling') or {}).get('factor', 1.0))
         s.window, s.keep_first = int(mask.get('size', 0)), int(mask.get('keep_first', 0))
         if s.rot_dims % 2 or not 0 <= s.rot_dims <= s.dim or s.rot_scale <= 0:
             raise ValueError(f'layer {i}: rot.dims must be even and at most dim, the scaling factor positive')
     elif kind == 'lightning':
-        s.mixer, s.kv_heads, s.vdim = MIXER_LIGHTNING, s.heads, int(m['vdim'])
+        s.mixer, s.kv_heads, s.vdim = MIXER_LIGHTNING, s.heads, int(m.get('vdim', s.dim))
         d = m['decay']
         s.decay = tuple(float(v) for v in d) if isinstance(d, (list, tuple)) else (float(d),) * s.heads
         if len(s.decay) != s.heads:

@@ -79,7 +79,8 @@ def windowed_attention(q, k, v, scale, window, keep_first, pos0=0):
 
 def attention_mixer(h, m, w, p, eps):
     T = h.shape[0]
-    H, G, d, dv = m['heads'], m['kv_heads'], m['dim'], m['vdim']
+    H, d = m['heads'], m['dim']
+    G, dv = m.get('kv_heads', H), m.get('vdim', d)
     q = (h @ w[p + 'q'].T + w[p + 'q.b']).reshape(T, H, d)
     k = (h @ w[p + 'k'].T + w[p + 'k.b']).reshape(T, G, d)
     v = (h @ w[p + 'v'].T + w[p + 'v.b']).reshape(T, G, dv)
@@ -87,9 +88,10 @@ def attention_mixer(h, m, w, p, eps):
     rot, mask = m.get('rot') or {}, m.get('mask') or {}
     factor = float((rot.get('scaling') or {}).get('factor', 1.0))
     pos = np.arange(T)
-    q = rotate(q, pos, int(rot.get('dims', 0)), float(rot.get('base', 10000.0)), factor)
-    k = rotate(k, pos, int(rot.get('dims', 0)), float(rot.get('base', 10000.0)), factor)
-    o = windowed_attention(q, k, v, m['scale'], int(mask.get('size', 0)), int(mask.get('keep_first', 0)))
+    dims = int(rot.get('dims', d)) if rot else 0
+    q = rotate(q, pos, dims, float(rot.get('base', 10000.0)), factor)
+    k = rotate(k, pos, dims, float(rot.get('base', 10000.0)), factor)
+    o = windowed_attention(q, k, v, m.get('scale', d ** -0.5), int(mask.get('size', 0)), int(mask.get('keep_first', 0)))
     return o.reshape(T, H * dv) @ w[p + 'o'].T
 
 
