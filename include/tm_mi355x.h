@@ -505,7 +505,7 @@ int tm_gemm_export(const char* path);
  * Norms, attention scores and weights, and the residual sum are fp32 in both.
  * Weight slots (tm_engine_weight_copy, checkpoint bytes: bf16, [out][in]): "embed", "l<i>.norm1", "l<i>.norm2" (with an ff),
  * "l<i>.mix.q|k|v|o", "l<i>.mix.sink" (with a sink), "l<i>.mlp.up|down", "final.norm", "head". */
-enum { TM_MIXER_ATTENTION = 1, TM_MIXER_LATENT = 2, TM_MIXER_LIGHTNING = 3, TM_MIXER_DELTA = 4 };
+enum { TM_MIXER_ATTENTION = 1, TM_MIXER_LATENT = 2, TM_MIXER_LIGHTNING = 3, TM_MIXER_DELTA = 4, TM_MIXER_PARALLEL = 5 };
 enum { TM_MLP_NONE = 0, TM_MLP_DENSE = 1, TM_MLP_GATED = 2, TM_MLP_MOE = 3 };
 enum { TM_ACT_RELU2 = 0, TM_ACT_GELU_TANH = 1, TM_ACT_SILU = 2, TM_ACT_XIELU = 3 };
 enum { TM_DTYPE_BF16 = 0, TM_DTYPE_F32 = 1 };
@@ -564,6 +564,37 @@ typedef struct tm_layer_spec {
     int          expert_plain, router_softmax;
     float        router_scale;
     int          shared_ff;
+    /* further switches of post_norm blocks (all off at 0):
+     *   norm_groups > 0: the norm behind a sublayer is an RMS norm in that many equal consecutive groups of the row, times "norm<i>" (no bias,
+     *     no mean) instead of the layer norm.  TM_MLP_GATED (act TM_ACT_SILU | TM_ACT_GELU_TANH | TM_ACT_RELU2) is then allowed as feed-forward.
+     *   conv_taps > 0: every channel of the q, k, v projections passes a causal convolution over time ("mix.q.conv" [channels][taps], the last
+     *     column meets the current token, zeros before the sequence) ahead of norm and rotation; the last taps - 1 projected rows are state.
+     *   diff_maps: differential attention -- queries and keys hold two maps per head ([map 1 | map 2], 2 dim channels per head), each an
+     *     attention over the same values; o = a1 - lambda a2, lambda = exp(lq1 . lk1) - exp(lq2 . lk2) + diff_init ("mix.lq1" ... [dim]),
+     *     o scaled to unit RMS per head, times 1 - diff_init.
+     *   rot_pairs: the rotation pairs channel 2i with 2i + 1 instead of i with i + rot_dims / 2.
+     *   yarn_factor > 0: frequencies f_i = base^(-2i / rot_dims) become f_i / factor * r_i + f_i (1 - r_i), r_i = clamp((i - lo) / max(hi - lo,
+     *     0.001), 0, 1), lo = max(floor(c(yarn_fast)), 0), hi = min(ceil(c(yarn_slow)), rot_dims - 1), c(t) = rot_dims ln(yarn_original /
+     *     (2 pi t)) / (2 ln base); cos and sin are multiplied by 0.1 ln(factor) + 1.
+     *   TM_MIXER_PARALLEL: two mixers read the block's input; the result is half the sum of their outputs, each RMS-normed over the width
+     *     with "mix.left.out" / "mix.right.out".
+     *     left ("mix.left.*", sizes heads / kv_heads / dim / vdim, scale, window): attention without rotation whose values are the keys as
+     *       projected (vdim = dim, no "v"); queries and keys RMS-normed over the WHOLE projection with weights "q.norm" / "k.norm"; the
+     *       score gets "rel"[bucket(distance)][head] (dist_buckets rows: one per distance below half of them, logarithmic up to dist_max
+     *       above), then the heads' scores are mixed by "talk" [heads][heads]; one is added to the soft-max denominator; the
+     *       concatenated heads are multiplied by sigmoid("g" x) ahead of "o".
+     *     right ("mix.right.*", sizes r_heads / r_kv_heads / r_dim / r_vdim): gated delta rule.  q, k ([r_kv_heads][r_dim]) and v
+     *       ([r_heads][r_vdim]) pass a convolution of r_conv taps and silu; q, k become unit vectors per head (q also times r_dim^-1/2);
+     *       beta = sigmoid("b" x) per head; decay g = exp(-exp(A_log[head]) softplus(a2 (a1 x) + dt_bias)) per head and key channel;
+     *       S <- diag(g) S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q; every head's o scaled to unit RMS, times "norm" [r_vdim],
+     *       times sigmoid(g2 (g1 x)); then "o".  a_rank / g_rank = rows of "a1" / "g1". */
+    int          norm_groups, conv_taps, diff_maps;
+    float        diff_init;
+    int          rot_pairs;
+    float        yarn_factor, yarn_original, yarn_fast, yarn_slow;
+    int          dist_buckets;
+    float        dist_max;
+    int          r_heads, r_kv_heads, r_dim, r_vdim, r_conv, a_rank, g_rank;
 } tm_layer_spec;
 typedef struct tm_layered_config {
     int                  width, vocab, n_layers;
@@ -572,6 +603,9 @@ typedef struct tm_layered_config {
     int                  dtype;
     int                  loop_times; /* 0: no loop tensors */
     int                  final_layer_norm; /* != 0: the model's last norm is a layer norm with bias ("final.norm", "final.norm.b") */
+    float                embed_scale;      /* the embedding output is multiplied by it (0: 1) */
+    float                logit_softcap;    /* > 0: logits <- cap * tanh(logits / cap) */
+    int                  norm_groups;      /* > 0: the model's last norm is an RMS norm in that many groups ("final.norm") */
 } tm_layered_config;
 /* cfg->model is ignored; tp must be 1; quant_policy 0 (the cache holds the activation type) */
 int tm_engine_create_layered(tm_engine** out, const tm_engine_config* cfg, const tm_layered_config* model);
@@ -643,6 +677,12 @@ typedef struct tm_general_attn {
     int             ld_gate, out_head_stride;
     /* window > 0: a row at position i sees key j <= i only if i - j < window or j < keep_first */
     int             window, keep_first;
+    /* k_heads / v_heads > 0: the cache holds that many key / value heads; the query heads form kv_heads groups, group g reads key head
+     * g % k_heads and value head g % v_heads (0: kv_heads of each).  dist_table [q_heads][dist_table_len] fp32: the score gets
+     * dist_table[head][min(distance, len - 1)].  out_f32: the output rows are fp32 whatever the cache holds */
+    int             k_heads, v_heads;
+    const float*    dist_table;
+    int             dist_table_len, out_f32;
 } tm_general_attn;
 size_t tm_general_attention_workspace(int rows, int q_heads, int vdim, int splits);
 int    tm_general_attention(const tm_general_attn* a, tm_stream_t st);

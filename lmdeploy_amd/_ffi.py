@@ -76,14 +76,18 @@ class LayerSpec(C.Structure):
                 ('kv_rank', c_int), ('rot_dim', c_int), ('rot_base', c_float), ('experts', c_int), ('top', c_int), ('rot_dims', c_int),
                 ('post_norm', c_int), ('qkv_bias', c_int), ('qk_norm_w', c_int), ('rot_scale', c_float), ('window', c_int),
                 ('keep_first', c_int), ('decay', POINTER(c_float)), ('decay_rank', c_int), ('expert_plain', c_int),
-                ('router_softmax', c_int), ('router_scale', c_float), ('shared_ff', c_int)]
+                ('router_softmax', c_int), ('router_scale', c_float), ('shared_ff', c_int),
+                ('norm_groups', c_int), ('conv_taps', c_int), ('diff_maps', c_int), ('diff_init', c_float), ('rot_pairs', c_int),
+                ('yarn_factor', c_float), ('yarn_original', c_float), ('yarn_fast', c_float), ('yarn_slow', c_float),
+                ('dist_buckets', c_int), ('dist_max', c_float), ('r_heads', c_int), ('r_kv_heads', c_int), ('r_dim', c_int),
+                ('r_vdim', c_int), ('r_conv', c_int), ('a_rank', c_int), ('g_rank', c_int)]
 
 
 class LayeredConfig(C.Structure):
     """struct tm_layered_config"""
     _fields_ = [('width', c_int), ('vocab', c_int), ('n_layers', c_int), ('layers', POINTER(LayerSpec)), ('norm_eps', c_float),
                 ('norm_offset', c_float), ('residual_mult', c_float), ('logit_scale', c_float), ('dtype', c_int), ('loop_times', c_int),
-                ('final_layer_norm', c_int)]
+                ('final_layer_norm', c_int), ('embed_scale', c_float), ('logit_softcap', c_float), ('norm_groups', c_int)]
 
 
 class StepEntry(C.Structure):
@@ -100,7 +104,8 @@ class GeneralAttn(C.Structure):
                 ('splits', c_int), ('workspace', c_void_p), ('kv', c_void_p), ('ldkv', c_int), ('k_col', c_int), ('v_col', c_int),
                 ('store_kv', c_int), ('kernel', c_int), ('prefill', c_int), ('nseq', c_int), ('max_q_len', c_int), ('cu_q', c_void_p),
                 ('k_len', c_void_p), ('dist_r1', c_void_p), ('dist_r2', c_void_p), ('chunk', c_int), ('out_gate', c_void_p),
-                ('ld_gate', c_int), ('out_head_stride', c_int), ('window', c_int), ('keep_first', c_int)]
+                ('ld_gate', c_int), ('out_head_stride', c_int), ('window', c_int), ('keep_first', c_int), ('k_heads', c_int),
+                ('v_heads', c_int), ('dist_table', c_void_p), ('dist_table_len', c_int), ('out_f32', c_int)]
 
 
 # name -> (restype, argtypes); every int-returning function is a tm_status

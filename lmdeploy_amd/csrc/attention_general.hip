@@ -10,7 +10,11 @@
 //   * output gate:                   head h of row t is multiplied by sigmoid(out_gate[t][h])        (out_gate = nullptr: off)
 //   * sliding window:                a row at position p sees key j <= p only if p - j < window or j < keep_first: the window plus
 //                                    the first tokens of the sequence, at their true positions             (window = 0: off)
-// Scores, soft-max weights and the output accumulation are fp32 whatever the cache holds.
+//   * distance table:                score += dist_table[head][min(p - key position, len - 1)]: a learned bias per distance (a bucketed
+//                                    table is expanded per distance by the caller)                   (dist_table = nullptr: off)
+//   * key / value head counts of their own: the query heads form kv_heads groups; group g reads key head g % k_heads and value head
+//                                    g % v_heads (two score maps over one set of values; one wide key with a value head per group)
+// Scores, soft-max weights and the output accumulation are fp32 whatever the cache holds; out_f32 keeps the output rows in fp32 too.
 //
 // One launch serves every row of a forward, prefill portions and decoded tokens alike: row t belongs to sequence row_seq[t] at
 // position row_pos[t] and sees the cache entries 0 .. row_pos[t] of that sequence (its own key was stored before the launch).
@@ -133,6 +137,29 @@ __device__ __forceinline__ float ga_out_gate(const GeneralAttnParams& p, int t, 
     return p.out_gate ? 1.f / (1.f + expf(-p.out_gate[(size_t)t * p.ld_gate + h])) : 1.f;
 }
 
+// key / value head of a group of query heads
+__device__ __forceinline__ int ga_key_head(const GeneralAttnParams& p, int g)
+{
+    return p.k_heads > 0 ? g % p.k_heads : g;
+}
+__device__ __forceinline__ int ga_value_head(const GeneralAttnParams& p, int g)
+{
+    return p.v_heads > 0 ? g % p.v_heads : g;
+}
+
+// channel v of head h of output row t
+template<class T>
+__device__ __forceinline__ void ga_store(const GeneralAttnParams& p, int t, int h, int v, float val)
+{
+    const size_t at = (size_t)t * p.ldo + ga_out_head(p, h) + v;
+    if (p.out_f32) {
+        ((float*)p.out)[at] = val;
+    }
+    else {
+        ((T*)p.out)[at] = (T)val;
+    }
+}
+
 // grid (rows, ceil(q_heads / 4), splits), 256 threads: wave w -> head blockIdx.y * 4 + w
 template<class T, int VC>
 __global__ __launch_bounds__(256) void attn_rows_kernel(GeneralAttnParams p)
@@ -170,8 +197,8 @@ __global__ __launch_bounds__(256) void attn_rows_kernel(GeneralAttnParams p)
     for (int bi = i0; bi < i1; ++bi) {
         const int   b    = ga_block_at(bi, nk, bf);
         const char* base = (const char*)table[b] + p.layer_offset;
-        const T*    kb   = (const T*)base + (size_t)g * p.block_len * D;
-        const T*    vb   = (const T*)(base + p.v_offset) + (size_t)g * p.block_len * V;  // [V][block_len]
+        const T*    kb   = (const T*)base + (size_t)ga_key_head(p, g) * p.block_len * D;
+        const T*    vb   = (const T*)(base + p.v_offset) + (size_t)ga_value_head(p, g) * p.block_len * V;  // [V][block_len]
         const int   n    = min(p.block_len, nkeys - b * p.block_len);
         const int   jlo  = first - b * p.block_len;  // keys below it lie in an earlier chunk / before the window ...
         const int   klo  = keep - b * p.block_len;   // ... and are seen only as kept first tokens: j < klo
@@ -183,6 +210,9 @@ __global__ __launch_bounds__(256) void attn_rows_kernel(GeneralAttnParams p)
                 sc = ga_modify(p, ga_dot<T>(kb + (size_t)j * D, qs[wave], D), qscale);
                 if (p.dist_r1) {
                     sc -= r1 * log1pf(r2 * (float)(pos - (b * p.block_len + j)));
+                }
+                if (p.dist_table) {
+                    sc += p.dist_table[(size_t)h * p.dist_table_len + min(pos - (b * p.block_len + j), p.dist_table_len - 1)];
                 }
             }
             const float m_new = fmaxf(m, ga_wave_max(sc));
@@ -218,12 +248,11 @@ __global__ __launch_bounds__(256) void attn_rows_kernel(GeneralAttnParams p)
             inv = 1.f / l;
         }
         inv *= ga_out_gate(p, t, h);
-        T* out = (T*)p.out + (size_t)t * p.ldo + ga_out_head(p, h);
 #pragma unroll
         for (int c = 0; c < VC; ++c) {
             const int v = lane + 64 * c;
             if (v < V) {
-                out[v] = (T)(o[c] * inv);
+                ga_store<T>(p, t, h, v, o[c] * inv);
             }
         }
         return;
@@ -272,12 +301,11 @@ __global__ __launch_bounds__(64) void attn_rows_merge_kernel(GeneralAttnParams p
         }
     }
     const float inv = ga_out_gate(p, t, h) / l;
-    T* out = (T*)p.out + (size_t)t * p.ldo + ga_out_head(p, h);
 #pragma unroll
     for (int c = 0; c < VC; ++c) {
         const int v = lane + 64 * c;
         if (v < V) {
-            out[v] = (T)(o[c] * inv);
+            ga_store<T>(p, t, h, v, o[c] * inv);
         }
     }
 }
@@ -315,6 +343,7 @@ int launch_general_attention_rows(const GeneralAttnParams& p, hipStream_t st)
     TM_REQUIRE(p.dim >= 1 && p.dim <= kGaMaxDim && p.vdim >= 1 && p.vdim <= kGaMaxDim, "attention: 1 <= dim, vdim <= 1024");
     TM_REQUIRE(p.chunk >= 0 && (!p.dist_r1 || p.dist_r2) && (!p.out_gate || p.ld_gate >= p.q_heads), "attention: chunk / distance penalty / gate");
     TM_REQUIRE(p.window >= 0 && p.keep_first >= 0, "attention: window / kept first tokens");
+    TM_REQUIRE(p.k_heads >= 0 && p.v_heads >= 0 && (!p.dist_table || p.dist_table_len >= 1), "attention: key / value head counts, distance table");
     TM_REQUIRE(p.block_len >= 1 && p.splits >= 1 && (p.splits == 1 || (p.partial_o && p.partial_ml)), "attention: splits / workspace");
     TM_REQUIRE(p.elem_bytes == 2 || p.elem_bytes == 4, "attention: bf16 or fp32");
     TM_REQUIRE(p.qtemp_coef == 0.f || p.qtemp_every > 0.f, "attention: query temperature period");
@@ -364,12 +393,13 @@ __device__ __forceinline__ float ga_tanh_fast(float x)
 // (block-relative; < 0: none); kb / vb: the key head's keys [64][D] and transposed values [V][64] of this block.
 // lower: first key of the visible range of the lane's rows (block-relative, may be negative); keys below it are seen while < keep_rel
 // (the kept first tokens, block-relative; <= 0: none); r1 / r2: the distance penalty of the lane's rows' head
-// (r1 * log2(1 + r2 * (limit - key)) leaves the score, which lives in the log2 domain; bias = false: none)
+// (r1 * log2(1 + r2 * (limit - key)) leaves the score, which lives in the log2 domain; bias = false: none); tab: the distance table's row
+// of the lane's rows' head (nullptr: none)
 template<int DS, int VT, int RT, bool MASK, bool EAGER>
 __device__ __forceinline__ void ga_block_step(const bf16x8 (&qf)[RT][DS], const __bf16* __restrict__ kb, const __bf16* __restrict__ vb, int D,
                                               int V, const int (&limit)[RT], const int (&lower)[RT], int keep_rel, const float (&qscale)[RT], float cap,
                                               float inv_cap, bool bias, float r1, float r2, float (&m)[RT], float (&l)[RT],
-                                              floatx4 (&o)[RT][VT])
+                                              floatx4 (&o)[RT][VT], const float* __restrict__ tab = nullptr, int tab_len = 0)
 {
     const int    lane = threadIdx.x & 63, lr = lane & 15, lg = lane >> 4;
     const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -438,6 +468,9 @@ __device__ __forceinline__ void ga_block_step(const bf16x8 (&qf)[RT][DS], const 
                 if (bias) {  // (a key ahead of the row gives the logarithm of a number that may be negative: the mask below discards it)
                     v = fmaf(-r1, __builtin_amdgcn_logf(fmaf(r2, (float)(limit[rt] - key), 1.f)), v);
                 }
+                if (tab) {  // the lane's head's row of the distance table (a key ahead of the row reads entry 0 and is masked below)
+                    v = fmaf(tab[min(max(limit[rt] - key, 0), tab_len - 1)], kLog2e, v);
+                }
                 if (MASK) {
                     v = (key <= limit[rt] && (key >= lower[rt] || key < keep_rel)) ? v : -1e30f;
                 }
@@ -505,6 +538,7 @@ __global__ __launch_bounds__(256) void attn_tiles_kernel(GeneralAttnParams p, in
     int     pos[RT], first[RT];
     const bool  bias = p.dist_r1 != nullptr;
     const float r1 = bias ? p.dist_r1[h] : 0.f, r2 = bias ? p.dist_r2[h] : 0.f;
+    const float* tab = p.dist_table ? p.dist_table + (size_t)h * p.dist_table_len : nullptr;
     bool    q_ok[RT];
     floatx4 o[RT][VT];
 #pragma unroll
@@ -541,13 +575,15 @@ __global__ __launch_bounds__(256) void attn_tiles_kernel(GeneralAttnParams p, in
             limit[rt] = q_ok[rt] ? pos[rt] - b * 64 : -1;
             lower[rt] = first[rt] - b * 64;
         }
-        const __bf16 *kb = (const __bf16*)base + (size_t)g * 64 * D, *vb = (const __bf16*)(base + p.v_offset) + (size_t)g * 64 * V;
+        const __bf16 *kb = (const __bf16*)base + (size_t)ga_key_head(p, g) * 64 * D;
+        const __bf16 *vb = (const __bf16*)(base + p.v_offset) + (size_t)ga_value_head(p, g) * 64 * V;
         // every row of the wave sees the whole block (rows beyond the portion are discarded anyway)
         if (b * 64 + 63 <= pos0 + row0 && b * 64 >= first_hi) {
-            ga_block_step<DS, VT, RT, false, false>(qf, kb, vb, D, V, limit, lower, 0, qscale, cap, inv_cap, bias, r1, r2, m, l, o);
+            ga_block_step<DS, VT, RT, false, false>(qf, kb, vb, D, V, limit, lower, 0, qscale, cap, inv_cap, bias, r1, r2, m, l, o, tab, p.dist_table_len);
         }
         else {
-            ga_block_step<DS, VT, RT, true, false>(qf, kb, vb, D, V, limit, lower, keep - b * 64, qscale, cap, inv_cap, bias, r1, r2, m, l, o);
+            ga_block_step<DS, VT, RT, true, false>(qf, kb, vb, D, V, limit, lower, keep - b * 64, qscale, cap, inv_cap, bias, r1, r2, m, l, o, tab,
+                                                   p.dist_table_len);
         }
     }
 #pragma unroll
@@ -565,14 +601,13 @@ __global__ __launch_bounds__(256) void attn_tiles_kernel(GeneralAttnParams p, in
         }
         inv *= ga_out_gate(p, row_base + row0 + rt * 16 + lr, h);
         // lane holds O[row lr][channel t * 16 + lg * 4 + r]
-        __bf16* out = (__bf16*)p.out + (size_t)(row_base + row0 + rt * 16 + lr) * p.ldo + ga_out_head(p, h);
 #pragma unroll
         for (int t = 0; t < VT; ++t) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int v = t * 16 + lg * 4 + r;
                 if (v < V) {
-                    out[v] = (__bf16)(o[rt][t][r] * inv);
+                    ga_store<__bf16>(p, row_base + row0 + rt * 16 + lr, h, v, o[rt][t][r] * inv);
                 }
             }
         }
@@ -616,6 +651,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(GeneralAttnParams p, i
     }
     const bool  bias = p.dist_r1 != nullptr;
     const float r1 = bias ? p.dist_r1[h] : 0.f, r2 = bias ? p.dist_r2[h] : 0.f;  // of the lane's head
+    const float* tab = p.dist_table ? p.dist_table + (size_t)h * p.dist_table_len : nullptr;
     const int first = ga_first_key(p, pos), bf = first / 64;
     const int keep = ga_keep(p), nk = ga_keep_blocks(p, first, bf, 64);
     const int nvis = nk + pos / 64 + 1 - bf, per = (nvis + p.splits - 1) / p.splits;
@@ -624,8 +660,9 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(GeneralAttnParams p, i
         const int   b    = ga_block_at(bi, nk, bf);
         const char* base = (const char*)table[b] + p.layer_offset;
         const int limit[1] = {pos - b * 64}, lower[1] = {first - b * 64};
-        ga_block_step<DS, VT, 1, true, true>(qf, (const __bf16*)base + (size_t)g * 64 * D, (const __bf16*)(base + p.v_offset) + (size_t)g * 64 * V, D,
-                                       V, limit, lower, keep - b * 64, qscale, cap, inv_cap, bias, r1, r2, m1, l1, o1);
+        ga_block_step<DS, VT, 1, true, true>(qf, (const __bf16*)base + (size_t)ga_key_head(p, g) * 64 * D,
+                                             (const __bf16*)(base + p.v_offset) + (size_t)ga_value_head(p, g) * 64 * V, D, V, limit, lower,
+                                             keep - b * 64, qscale, cap, inv_cap, bias, r1, r2, m1, l1, o1, tab, p.dist_table_len);
     }
     const float m = m1[0] * kLn2, l = l1[0];  // back from the log2 domain: the merge below and the split merge kernel use e^x
     floatx4 (&o)[VT] = o1[0];
@@ -673,14 +710,13 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(GeneralAttnParams p, i
             inv = 1.f / lt;
         }
         inv *= ga_out_gate(p, t, h);
-        __bf16* out = (__bf16*)p.out + (size_t)t * p.ldo + ga_out_head(p, h);
 #pragma unroll
         for (int v = 0; v < VT; ++v) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int c = v * 16 + lg * 4 + r;
                 if (c < V) {
-                    out[c] = (__bf16)(o[v][r] * inv);
+                    ga_store<__bf16>(p, t, h, c, o[v][r] * inv);
                 }
             }
         }

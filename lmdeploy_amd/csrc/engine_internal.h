@@ -99,6 +99,23 @@ struct LmLayer {
     float *            w0 = nullptr, *act_par = nullptr, *decay_d = nullptr;
     std::vector<float> decay_h;                 // lightning: the spec's decays (the spec's pointer is the caller's memory)
     size_t             state_offset = 0, state_floats = 0;  // this layer run's state inside a slot of the state pool (floats)
+    // post-norm blocks with RMS group norms (spec.norm_groups): convolved projections, differential attention, and the parallel pair of a
+    // biased attention (left) and a gated delta rule (right).  Fused projection columns
+    //   attention: [q | k | v]                                 (two maps per query / key head with diff_maps)
+    //   parallel:  [left q | left k | left gate | right q | right k | right v | beta | a1 (padded to 32) | g1]
+    int          a_heads = 0;                  // query heads the attention kernel sees (two per head with diff_maps)
+    int          a_kh = 0, a_vh = 0;           // key / value heads in the cache where they differ from a_kv (0: a_kv of each)
+    bool         has_cache = true, has_state = false;
+    int          conv_col = 0, conv_ch = 0, conv_taps = 0, conv_act = 0;  // the projection columns [conv_col, conv_col + conv_ch) pass a convolution
+    float*       conv_w = nullptr;             // [conv_ch][taps]
+    size_t       conv_offset = 0, conv_floats = 0;  // its state inside a slot of the state pool
+    float *      lambda = nullptr, *dist_tab = nullptr, *talk = nullptr, *zero_sink = nullptr, *join_l = nullptr, *join_r = nullptr;
+    int          dist_len = 0;
+    int          c_rq = 0, c_rk = 0, c_rv = 0, c_b = 0, c_a1 = 0, c_g1 = 0;  // parallel: columns of the right mixer's projections
+    int          c_xq = 0, c_xk = 0;           // ... and of its per-head query / key vectors behind the convolved columns
+    int          r_nqk = 0, r_nv = 0, lora_g1 = 0;  // right: kv_heads * dim, heads * vdim; column of g1 among the cast inner activations
+    DenseWeight  wo_r, a2, g2;
+    float *      a_log = nullptr, *dt_bias = nullptr, *r_norm = nullptr;
 };
 
 struct LayeredModel {
@@ -121,6 +138,8 @@ struct LayeredModel {
     int *                d_topk_ids = nullptr, *d_offsets = nullptr, *d_f2n = nullptr, *d_en2f = nullptr;
     // post-norm blocks: a sublayer's fp32 result, state mixers' fp32 output and per-row vectors, the decay's inner activations
     float *              d_y = nullptr, *d_mixo = nullptr, *d_aux = nullptr, *d_wdec = nullptr, *final_norm_b = nullptr;
+    float *              d_y2 = nullptr, *d_conv = nullptr, *d_gate2 = nullptr;  // the second branch's result, convolved projections, a gate
+    int                  ldconv = 0;
     void*                d_lora = nullptr;
     int                  ldmix = 0, ldlora = 0;
     // recurrent states: [max_batch_size + 1 slots][state_slot_floats] fp32; the last slot takes the decode rows of slots without a sequence

@@ -31,6 +31,17 @@
 //   y        = cat . Wo^T (fp32);   x += LN1(y), h = x            one launch
 //   dense:   y = down(xielu(up h));   experts: soft-max router top-k -> rows sorted by expert -> two batched products -> weighted sum
 //            (+ the shared expert);   x += LN2(y), h = x
+//
+// Post-norm blocks with RMS group norms (spec.norm_groups > 0; group_layer()): x += GN1(mixer(x)); x += GN2(ff(x)),
+//   proj     = h . [every projection of the mixer]^T               ONE GEMM, fp32 output
+//   conv     = short causal convolution of the q, k, v columns (its last inputs live in the slot's state)      launch_short_conv
+//   differential attention:  launch_attn_prep (two maps per head leave as heads of their own; norm, pairwise rotation) -> attention over
+//            2 G key heads and G value heads, fp32 output -> o = a1 - lambda a2, unit RMS per head (launch_diff_head_norm) -> Wo
+//   parallel: left  = launch_talk_prep (norms over the whole projection; the head-mixing matrix folded into the queries) -> attention over
+//                     one wide key with a distance table and a zero sink -> sigmoid gate -> Wo (left)
+//             right = conv + silu -> decay / gate inner products -> launch_gdelta_prep -> launch_state_mix -> gated head norm -> Wo (right)
+//             x += GN1(0.5 (rms(left) w_l + rms(right) w_r)), h = x                                              one launch
+//   gated feed-forward: act(gate h) * (up h) in the epilogue of ONE product, down; x += GN2(y), h = x
 #include "engine_internal.h"
 
 namespace tmk {
@@ -68,6 +79,21 @@ __global__ void bf16_to_f32_kernel(float* out, const uint16_t* in, size_t n)
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) {
         out[i] = __builtin_bit_cast(float, (uint32_t)in[i] << 16);
+    }
+}
+
+// lambda of differential attention: exp(lq1 . lk1) - exp(lq2 . lk2) + init, from the checkpoint's bf16 vectors
+__global__ void diff_lambda_kernel(float* out, const uint16_t* q1, const uint16_t* k1, const uint16_t* q2, const uint16_t* k2, int n, float init)
+{
+    auto f = [](uint16_t b) { return __builtin_bit_cast(float, (uint32_t)b << 16); };
+    float a = 0.f, b = 0.f;
+    for (int i = threadIdx.x; i < n; i += 64) {
+        a = fmaf(f(q1[i]), f(k1[i]), a);
+        b = fmaf(f(q2[i]), f(k2[i]), b);
+    }
+    a = group_sum<64>(a), b = group_sum<64>(b);
+    if (threadIdx.x == 0) {
+        out[0] = expf(a) - expf(b) + init;
     }
 }
 
@@ -195,9 +221,177 @@ static int to_f32_at(tm_engine* e, const std::string& name, size_t n, float* out
     return 0;
 }
 
+// a bf16 vector / matrix of a slot on the host, as floats
+static int slot_to_host(tm_engine* e, const std::string& name, size_t n, std::vector<float>& out)
+{
+    Slot& s = e->slots[name];
+    TM_REQUIRE(s.filled && (int64_t)n * 2 <= s.bytes, "weight not loaded: " + name);
+    std::vector<uint16_t> raw(n);
+    TM_HIP_CHECK(hipStreamSynchronize(e->stream));
+    TM_HIP_CHECK(hipMemcpy(raw.data(), s.dev, n * 2, hipMemcpyDeviceToHost));
+    out.resize(n);
+    for (size_t i = 0; i < n; ++i) {
+        const uint32_t b = (uint32_t)raw[i] << 16;
+        memcpy(&out[i], &b, 4);
+    }
+    return 0;
+}
+
+static int upload_f32(tm_engine* e, const std::vector<float>& v, float** out)
+{
+    TM_TRY(dmalloc(out, std::max<size_t>(1, v.size())));
+    if (!v.empty()) {
+        TM_HIP_CHECK(hipMemcpy(*out, v.data(), v.size() * 4, hipMemcpyHostToDevice));
+    }
+    return 0;
+}
+
+// rotation frequencies of the first `dims` channels of a head; yarn_factor > 0: the slow frequencies are divided by it, with a linear ramp
+// between the channel that turns `fast` times over `original` positions and the one that turns `slow` times (see tm_layer_spec)
+static std::vector<float> rotation_frequencies(const tm_layer_spec& s)
+{
+    const int          dims = s.rot_dims;
+    std::vector<float> f(dims / 2);
+    const double       base = s.rot_base;
+    double             lo = 0, hi = 0;
+    if (s.yarn_factor > 0.f) {
+        auto dim_of = [&](double turns) { return dims * std::log((double)s.yarn_original / (2.0 * M_PI * turns)) / (2.0 * std::log(base)); };
+        lo = std::max(std::floor(dim_of(s.yarn_fast)), 0.0);
+        hi = std::min(std::ceil(dim_of(s.yarn_slow)), (double)dims - 1.0);
+    }
+    for (int j = 0; j < dims / 2; ++j) {
+        double v = std::pow(base, -2.0 * j / dims) / (double)s.rot_scale;
+        if (s.yarn_factor > 0.f) {
+            const double ramp = std::min(1.0, std::max(0.0, (j - lo) / std::max(hi - lo, 0.001)));
+            v                 = v / (double)s.yarn_factor * ramp + v * (1.0 - ramp);
+        }
+        f[j] = (float)v;
+    }
+    return f;
+}
+
+// post-norm blocks with RMS group norms: differential attention with convolved projections, or the parallel pair (see the head of this file)
+static int process_group_layer(tm_engine* e, int i, LmLayer& L, int dt)
+{
+    const tm_layer_spec& s = L.spec;
+    const int            W = e->lm->cfg.width, H = s.heads;
+    hipStream_t          st = e->stream;
+    TM_TRY(dense_weight_alloc(L.qkv, W, L.c_end, dt, st));
+    auto conv_weights = [&](const char* pre, int nq, int nk, int nv, int taps) -> int {
+        TM_TRY(dmalloc(&L.conv_w, (size_t)(nq + nk + nv) * taps));
+        TM_TRY(to_f32_at(e, lname(i, (std::string(pre) + "q.conv").c_str()), (size_t)nq * taps, L.conv_w));
+        TM_TRY(to_f32_at(e, lname(i, (std::string(pre) + "k.conv").c_str()), (size_t)nk * taps, L.conv_w + (size_t)nq * taps));
+        TM_TRY(to_f32_at(e, lname(i, (std::string(pre) + "v.conv").c_str()), (size_t)nv * taps, L.conv_w + (size_t)(nq + nk) * taps));
+        return 0;
+    };
+    if (s.mixer == TM_MIXER_ATTENTION) {
+        TM_TRY(place(e, L.qkv, 0, 0, lname(i, "mix.q"), L.n_q, W));
+        TM_TRY(place(e, L.qkv, L.c_k, 0, lname(i, "mix.k"), L.n_k, W));
+        TM_TRY(place(e, L.qkv, L.c_v, 0, lname(i, "mix.v"), L.n_v, W));
+        if (s.qk_norm_w) {
+            TM_TRY(to_f32(e, lname(i, "mix.q.norm"), s.dim, &L.q_w));
+            TM_TRY(to_f32(e, lname(i, "mix.k.norm"), s.dim, &L.k_w));
+        }
+        if (s.rot_dims > 0) {
+            TM_TRY(upload_f32(e, rotation_frequencies(s), &L.inv_freq));
+        }
+        if (s.conv_taps > 0) {
+            TM_TRY(conv_weights("mix.", L.n_q, L.n_k, L.n_v, s.conv_taps));
+        }
+        if (s.diff_maps) {
+            TM_TRY(dmalloc(&L.lambda, (size_t)1));
+            const char* names[4] = {"mix.lq1", "mix.lk1", "mix.lq2", "mix.lk2"};
+            const uint16_t* v[4];
+            for (int j = 0; j < 4; ++j) {
+                Slot& sl = e->slots[lname(i, names[j])];
+                TM_REQUIRE(sl.filled, "weight not loaded: " + lname(i, names[j]));
+                v[j] = (const uint16_t*)sl.dev;
+            }
+            diff_lambda_kernel<<<1, 64, 0, st>>>(L.lambda, v[0], v[1], v[2], v[3], s.dim, s.diff_init);
+            TM_HIP_CHECK(hipGetLastError());
+        }
+        TM_TRY(dense_weight_alloc(L.wo, L.n_att, W, dt, st));
+        TM_TRY(place(e, L.wo, 0, 0, lname(i, "mix.o"), W, L.n_att));
+    }
+    else {  // parallel: [left q | left k | left gate | right q | right k | right v | beta | a1 | g1]
+        const int Hr = s.r_heads, dr = s.r_dim, dvr = s.r_vdim;
+        TM_TRY(place(e, L.qkv, 0, 0, lname(i, "mix.left.q"), L.n_q, W));
+        TM_TRY(place(e, L.qkv, L.c_k, 0, lname(i, "mix.left.k"), L.n_k, W));
+        TM_TRY(place(e, L.qkv, L.c_g, 0, lname(i, "mix.left.g"), L.n_att, W));
+        TM_TRY(place(e, L.qkv, L.c_rq, 0, lname(i, "mix.right.q"), L.r_nqk, W));
+        TM_TRY(place(e, L.qkv, L.c_rk, 0, lname(i, "mix.right.k"), L.r_nqk, W));
+        TM_TRY(place(e, L.qkv, L.c_rv, 0, lname(i, "mix.right.v"), L.r_nv, W));
+        TM_TRY(place(e, L.qkv, L.c_b, 0, lname(i, "mix.right.b"), Hr, W));
+        TM_TRY(place(e, L.qkv, L.c_a1, 0, lname(i, "mix.right.a1"), s.a_rank, W));
+        TM_TRY(place(e, L.qkv, L.c_g1, 0, lname(i, "mix.right.g1"), s.g_rank, W));
+        TM_TRY(to_f32(e, lname(i, "mix.left.q.norm"), L.n_q, &L.q_w));
+        TM_TRY(to_f32(e, lname(i, "mix.left.k.norm"), L.n_k, &L.k_w));
+        TM_TRY(to_f32(e, lname(i, "mix.left.talk"), (size_t)H * H, &L.talk));
+        {   // the distance bias after the head mixing, per head and distance: tab[h][d] = sum_g talk[h][g] rel[bucket(d)][g]
+            std::vector<float> rel, talk;
+            const int          B = s.dist_buckets, half = B / 2;
+            TM_TRY(slot_to_host(e, lname(i, "mix.left.rel"), (size_t)B * H, rel));
+            TM_TRY(slot_to_host(e, lname(i, "mix.left.talk"), (size_t)H * H, talk));
+            L.dist_len = s.window > 0 ? std::min(s.window, e->cfg.session_len) : e->cfg.session_len;
+            std::vector<float> tab((size_t)H * L.dist_len);
+            const double       span = std::log((double)s.dist_max / std::max(half, 1));
+            for (int d = 0; d < L.dist_len; ++d) {
+                int b = d;
+                if (d >= half) {
+                    b = half > 0 ? std::min(B - 1, half + (int)std::floor(std::log((double)d / half) / span * (B - half))) : B - 1;
+                }
+                for (int h = 0; h < H; ++h) {
+                    double acc = 0;
+                    for (int g = 0; g < H; ++g) {
+                        acc += (double)talk[(size_t)h * H + g] * (double)rel[(size_t)b * H + g];
+                    }
+                    tab[(size_t)h * L.dist_len + d] = (float)acc;
+                }
+            }
+            TM_TRY(upload_f32(e, tab, &L.dist_tab));
+        }
+        TM_TRY(upload_f32(e, std::vector<float>(H, 0.f), &L.zero_sink));
+        TM_TRY(dense_weight_alloc(L.wo, L.n_att, W, dt, st));
+        TM_TRY(place(e, L.wo, 0, 0, lname(i, "mix.left.o"), W, L.n_att));
+        TM_TRY(dense_weight_alloc(L.wo_r, L.r_nv, W, dt, st));
+        TM_TRY(place(e, L.wo_r, 0, 0, lname(i, "mix.right.o"), W, L.r_nv));
+        TM_TRY(dense_weight_alloc(L.a2, s.a_rank, Hr * dr, dt, st));
+        TM_TRY(place(e, L.a2, 0, 0, lname(i, "mix.right.a2"), Hr * dr, s.a_rank));
+        TM_TRY(dense_weight_alloc(L.g2, s.g_rank, L.r_nv, dt, st));
+        TM_TRY(place(e, L.g2, 0, 0, lname(i, "mix.right.g2"), L.r_nv, s.g_rank));
+        TM_TRY(to_f32(e, lname(i, "mix.right.A_log"), Hr, &L.a_log));
+        TM_TRY(to_f32(e, lname(i, "mix.right.dt_bias"), (size_t)Hr * dr, &L.dt_bias));
+        {   // the head norm's weight [vdim] is shared by the heads: one copy per head for the gated head norm
+            std::vector<float> nw, all;
+            TM_TRY(slot_to_host(e, lname(i, "mix.right.norm"), dvr, nw));
+            for (int h = 0; h < Hr; ++h) {
+                all.insert(all.end(), nw.begin(), nw.end());
+            }
+            TM_TRY(upload_f32(e, all, &L.r_norm));
+        }
+        TM_TRY(conv_weights("mix.right.", L.r_nqk, L.r_nqk, L.r_nv, s.r_conv));
+        TM_TRY(to_f32(e, lname(i, "mix.left.out"), W, &L.join_l));
+        TM_TRY(to_f32(e, lname(i, "mix.right.out"), W, &L.join_r));
+    }
+    TM_TRY(to_f32(e, lname(i, "norm1"), W, &L.norm1));
+    if (s.mlp) {
+        TM_TRY(to_f32(e, lname(i, "norm2"), W, &L.norm2));
+        TM_TRY(dense_weight_alloc(L.gu, W, dense_pair_rows(s.ff), dt, st));  // gate and up interleaved: the activation is the GEMM's epilogue
+        TM_TRY(place(e, L.gu, 0, 0, lname(i, "mlp.gate"), s.ff, W, 0, 0, false, 1));
+        TM_TRY(place(e, L.gu, 0, 0, lname(i, "mlp.up"), s.ff, W, 0, 0, false, 2));
+        TM_TRY(dense_weight_alloc(L.down, s.ff, W, dt, st));
+        TM_TRY(place(e, L.down, 0, 0, lname(i, "mlp.down"), W, s.ff));
+    }
+    TM_HIP_CHECK(hipStreamSynchronize(st));
+    return 0;
+}
+
 static int process_post_layer(tm_engine* e, int i, LmLayer& L, int dt)
 {
     const tm_layer_spec& s = L.spec;
+    if (s.norm_groups > 0) {
+        return process_group_layer(e, i, L, dt);
+    }
     const int            W = e->lm->cfg.width, H = s.heads, N = L.c_end;
     TM_TRY(dense_weight_alloc(L.qkv, W, N, dt, e->stream));
     TM_TRY(place(e, L.qkv, 0, 0, lname(i, s.mixer == TM_MIXER_DELTA ? "mix.r" : "mix.q"), L.n_q, W));
@@ -350,7 +544,7 @@ int layered_process_weights(tm_engine* e)
     TM_TRY(dense_weight_alloc(lm.head, W, c.vocab, dt, e->stream));
     TM_TRY(place(e, lm.head, 0, 0, "head", c.vocab, W));
     TM_TRY(to_f32(e, "final.norm", W, &lm.final_norm));
-    if (c.final_layer_norm) {
+    if (c.final_layer_norm && c.norm_groups == 0) {
         TM_TRY(to_f32(e, "final.norm.b", W, &lm.final_norm_b));
     }
     {
@@ -393,11 +587,14 @@ int layered_init_synthetic(tm_engine* e, uint64_t seed)
         const size_t        dot = n.rfind('.');
         const std::string   leaf = dot == std::string::npos ? n : n.substr(dot + 1);
         const bool          isnorm = n.find("norm") != std::string::npos;
-        const bool          vec = isnorm || leaf == "sink" || leaf == "r1" || leaf == "r2" || leaf == "b" || leaf == "step" || leaf == "w0" || leaf == "act";
+        const bool          join = leaf == "out" && (n.find("left.out") != std::string::npos || n.find("right.out") != std::string::npos);
+        const bool          vec = isnorm || join || leaf == "sink" || leaf == "r1" || leaf == "r2" || (leaf == "b" && n.find("right.b") == std::string::npos)
+                                  || leaf == "step" || leaf == "w0" || leaf == "act" || leaf == "lq1" || leaf == "lk1" || leaf == "lq2" || leaf == "lk2"
+                                  || leaf == "rel" || leaf == "A_log" || leaf == "dt_bias";
         // matrices: N(0, 1 / in_features) keeps every projection's output at the scale of its input; vectors: small, around zero (norm
         // weights around 1 - norm_offset; distance-penalty numbers positive)
         float stdv = 0.02f, mean = 0.f;
-        if (isnorm && leaf != "b") {
+        if ((isnorm && leaf != "b") || join) {
             mean = 1.f - lm.cfg.norm_offset;
         }
         else if (leaf == "r1" || leaf == "r2") {
@@ -451,28 +648,41 @@ int layered_start(tm_engine* e)
     int     max_qkv = 8, max_cat = 32, max_vdim = 0, max_heads = 0;
     int     max_proj = 0, max_q = 0, max_plain = 0, max_lat = 0, max_ff = 0;
     bool    any_moe = false;
-    int     max_mix = 0, max_lora = 0;
+    int     max_mix = 0, max_lora = 0, max_conv = 0;
+    bool    any_join = false;
     for (LmLayer& L : lm.layers) {
-        const bool stateful = L.spec.mixer == TM_MIXER_LIGHTNING || L.spec.mixer == TM_MIXER_DELTA;
-        if (stateful) {  // a recurrent state per slot instead of cache entries
+        const bool stateful = L.has_state;
+        const bool parallel = L.spec.mixer == TM_MIXER_PARALLEL;
+        if (stateful) {  // a recurrent state per slot (instead of cache entries, or beside them)
             L.state_offset = lm.state_slot_floats;
-            L.state_floats = state_mix_floats(L.spec.heads, L.spec.dim, L.spec.vdim);
+            L.state_floats = parallel ? state_mix_floats(L.spec.r_heads, L.spec.r_dim, L.spec.r_vdim) : state_mix_floats(L.spec.heads, L.spec.dim, L.spec.vdim);
             lm.state_slot_floats += L.state_floats;
-            max_mix  = std::max(max_mix, L.n_att);
-            max_lora = std::max(max_lora, L.w2.Kp);
+            max_mix  = std::max(max_mix, parallel ? std::max(L.r_nv, L.spec.r_heads * L.spec.r_dim) : L.n_att);
+            max_lora = std::max(max_lora, parallel ? L.lora_g1 + L.g2.Kp : L.w2.Kp);
         }
-        else {
+        if (L.conv_taps > 0) {  // the last taps - 1 inputs of a short convolution are state too
+            L.conv_offset = lm.state_slot_floats;
+            L.conv_floats = (size_t)(L.conv_taps - 1) * L.conv_ch;
+            lm.state_slot_floats += L.conv_floats;
+            max_conv = std::max(max_conv, L.conv_ch + (parallel ? 2 * L.spec.r_heads * L.spec.r_dim : 0));
+        }
+        if (L.has_cache) {
             L.kv_offset = off;
             L.v_offset  = (int64_t)L.n_k * c.cache_block_seq_len * lm.elem;
             off += (int64_t)(L.n_k + L.n_v) * c.cache_block_seq_len * lm.elem;
             off         = (off + 15) / 16 * 16;
             max_vdim    = std::max(max_vdim, L.a_vdim);
-            max_heads   = std::max(max_heads, L.spec.heads);
+            max_heads   = std::max(max_heads, L.a_heads);
+        }
+        if (L.post && L.spec.norm_groups > 0) {  // the attention output stays fp32 until the heads are joined / gated
+            max_mix  = std::max(max_mix, L.a_heads * L.a_vdim);
+            max_cat  = std::max(max_cat, L.wo_r.Kp);
+            any_join = any_join || parallel;
         }
         if (L.post) {
             max_cat  = std::max(max_cat, L.wo.Kp);
             max_proj = std::max(max_proj, std::max(L.qkv.N, L.spec.experts));
-            max_q    = std::max(max_q, stateful ? 0 : L.spec.heads * L.a_dim);
+            max_q    = std::max(max_q, L.has_cache ? L.a_heads * L.a_dim : 0);
             if (L.spec.mlp) {
                 max_ff     = std::max(max_ff, std::max(L.down.Kp, L.sh_down.Kp));
                 lm.max_top = std::max(lm.max_top, L.spec.mlp == TM_MLP_MOE ? L.spec.top + (L.shared_fused ? 1 : 0) : 1);
@@ -537,6 +747,14 @@ int layered_start(tm_engine* e)
         TM_TRY(lm_alloc(&lm.d_aux, T * lm.ldmix, st));
         TM_TRY(lm_alloc(&lm.d_wdec, T * lm.ldmix, st));
         TM_TRY(lm_alloc((char**)&lm.d_lora, T * lm.ldlora * lm.elem, st));
+        if (max_conv > 0) {
+            lm.ldconv = (max_conv + 3) / 4 * 4;
+            TM_TRY(lm_alloc(&lm.d_conv, T * lm.ldconv, st));
+        }
+        if (any_join) {
+            TM_TRY(lm_alloc(&lm.d_y2, T * m.width, st));
+            TM_TRY(lm_alloc(&lm.d_gate2, T * lm.ldmix, st));
+        }
     }
     if (lm.state_slot_floats > 0) {
         TM_TRY(lm_alloc(&lm.d_state, ((size_t)B + 1) * lm.state_slot_floats, st));
@@ -619,8 +837,10 @@ void layered_free(tm_engine* e)
             dense_weight_free(L.qkv), dense_weight_free(L.up), dense_weight_free(L.out);
             dense_weight_free(L.wo), dense_weight_free(L.gu), dense_weight_free(L.down), dense_weight_free(L.uk), dense_weight_free(L.uv);
             dense_weight_free(L.w2), dense_weight_free(L.router), dense_weight_free(L.sh_up), dense_weight_free(L.sh_down);
+            dense_weight_free(L.wo_r), dense_weight_free(L.a2), dense_weight_free(L.g2);
             for (float* p : {L.norm1, L.norm2, L.sink, L.r1, L.r2, L.rg1_b, L.rg2_b, L.c_norm, L.inv_freq, L.norm1_b, L.norm2_b, L.proj_bias,
-                             L.q_w, L.k_w, L.mix_norm, L.w0, L.act_par, L.decay_d}) {
+                             L.q_w, L.k_w, L.mix_norm, L.w0, L.act_par, L.decay_d, L.conv_w, L.lambda, L.dist_tab, L.talk, L.zero_sink, L.join_l,
+                             L.join_r, L.a_log, L.dt_bias, L.r_norm}) {
                 if (p) {
                     (void)hipFree(p);
                 }
@@ -629,7 +849,8 @@ void layered_free(tm_engine* e)
     }
     dense_weight_free(lm.head);
     dense_weight_free(lm.loop_in);
-    for (void* p : {(void*)lm.d_y, (void*)lm.d_mixo, (void*)lm.d_aux, (void*)lm.d_wdec, lm.d_lora, (void*)lm.d_state, (void*)lm.final_norm_b}) {
+    for (void* p : {(void*)lm.d_y, (void*)lm.d_mixo, (void*)lm.d_aux, (void*)lm.d_wdec, lm.d_lora, (void*)lm.d_state, (void*)lm.final_norm_b,
+                    (void*)lm.d_y2, (void*)lm.d_conv, (void*)lm.d_gate2}) {
         if (p) {
             (void)hipFree(p);
         }
@@ -670,7 +891,16 @@ static GeneralAttnParams attn_params(tm_engine* e, const LmLayer& L, const LmPar
             p.out_gate = lm.d_proj + (size_t)P.row0 * lm.ldproj + L.c_g;
             p.ld_gate  = lm.ldproj;
         }
+        if (L.post && L.spec.norm_groups > 0 && (L.spec.diff_maps || L.spec.mixer == TM_MIXER_PARALLEL)) {
+            p.out     = lm.d_mixo + (size_t)P.row0 * lm.ldmix;  // fp32 until the maps are joined / the gate is applied
+            p.ldo     = lm.ldmix;
+            p.out_f32 = 1;
+        }
     }
+    p.k_heads        = L.a_kh;
+    p.v_heads        = L.a_vh;
+    p.dist_table     = L.dist_tab;
+    p.dist_table_len = L.dist_len;
     p.dist_r1 = L.r1;
     p.dist_r2 = L.r2;
     p.chunk   = L.spec.chunk;
@@ -686,7 +916,7 @@ static GeneralAttnParams attn_params(tm_engine* e, const LmLayer& L, const LmPar
     p.v_offset     = L.v_offset;
     p.block_len    = e->cfg.cache_block_seq_len;
     p.elem_bytes   = lm.elem;
-    p.q_heads      = L.spec.heads;
+    p.q_heads      = L.a_heads;
     p.kv_heads     = L.a_kv;
     p.dim          = L.a_dim;
     p.vdim         = L.a_vdim;
@@ -694,7 +924,7 @@ static GeneralAttnParams attn_params(tm_engine* e, const LmLayer& L, const LmPar
     p.softcap      = L.spec.softcap;
     p.qtemp_coef   = L.spec.qtemp_coef;
     p.qtemp_every  = L.spec.qtemp_every;
-    p.sink         = L.sink;
+    p.sink         = L.sink ? L.sink : L.zero_sink;
     p.nseq         = P.nseq;
     p.max_q_len    = P.max_q_len;
     p.cu_q         = P.cu_q;
@@ -793,6 +1023,129 @@ static int wide_layer(tm_engine* e, const LmLayer& L, int M, const LmPart* parts
     return 0;
 }
 
+// the sequences of a part as the state kernels read them; the caller sets layer_offset
+static StateMixParams state_seqs(tm_engine* e, const LmPart& P)
+{
+    LayeredModel&  lm = *e->lm;
+    StateMixParams sp;
+    sp.max_q_len = P.decode ? 1 : std::max(1, P.max_q_len);
+    sp.nseq = P.nseq, sp.cu_q = P.cu_q, sp.k_len = P.k_len, sp.seq_slot = P.seq_slot, sp.slot0 = P.slot0, sp.active = P.active;
+    sp.park_slot   = e->cfg.max_batch_size;
+    sp.state       = lm.d_state;
+    sp.slot_stride = lm.state_slot_floats;
+    return sp;
+}
+
+static int run_attention_parts(tm_engine* e, const LmLayer& L, const LmPart* parts, int nparts)
+{
+    LayeredModel& lm = *e->lm;
+    for (int i = 0; i < nparts; ++i) {
+        const LmPart&     P = parts[i];
+        GeneralAttnParams p = attn_params(e, L, P);
+        if (P.decode && lm.decode_splits > 1 && general_attention_workspace_bytes(P.rows, L.a_heads, L.a_vdim, lm.decode_splits) <= lm.attn_ws_bytes) {
+            p.splits     = lm.decode_splits;
+            p.partial_o  = lm.d_attn_ws;
+            p.partial_ml = lm.d_attn_ws + (size_t)P.rows * L.a_heads * p.splits * L.a_vdim;
+        }
+        TM_PROF(P_ATTN, TM_TRY(launch_general_attention(p, !P.decode, e->stream)));
+    }
+    return 0;
+}
+
+// one post-norm block with RMS group norms over M rows (see the head of this file); lm.d_h1 holds the stream in the activation type
+static int group_layer(tm_engine* e, const LmLayer& L, int M, const LmPart* parts, int nparts)
+{
+    LayeredModel&            lm = *e->lm;
+    const tm_layered_config& m  = lm.cfg;
+    const tm_layer_spec&     s  = L.spec;
+    hipStream_t              st = e->stream;
+    const int                W = m.width, H = s.heads, groups = s.norm_groups;
+    TM_PROF(P_GEMM_QKV, TM_TRY(launch_dense_linear(L.qkv, lm.d_h1, lm.ldw, lm.d_proj, lm.ldproj, M, kDenseScaleF32, 1.f, st)));
+    if (L.conv_taps > 0) {
+        for (int i = 0; i < nparts; ++i) {
+            const LmPart&  P  = parts[i];
+            StateMixParams sp = state_seqs(e, P);
+            sp.layer_offset   = L.conv_offset;
+            TM_PROF(P_KV_STORE, TM_TRY(launch_short_conv(lm.d_conv + (size_t)P.row0 * lm.ldconv, lm.ldconv, lm.d_proj + (size_t)P.row0 * lm.ldproj, lm.ldproj,
+                                                         L.conv_col, L.conv_w, L.conv_ch, L.conv_taps, L.conv_act, sp, st)));
+        }
+    }
+    if (s.mixer == TM_MIXER_ATTENTION) {
+        const float* src = L.conv_taps > 0 ? lm.d_conv : lm.d_proj;  // (the convolved columns start at column 0 of both)
+        const int    ld  = L.conv_taps > 0 ? lm.ldconv : lm.ldproj;
+        AttnPrepExtra ex;
+        ex.q_w = L.q_w, ex.k_w = L.k_w, ex.inv_freq = L.inv_freq, ex.rot_dims = s.rot_dims;
+        ex.maps = s.diff_maps ? 2 : 1, ex.rot_pairs = s.rot_pairs;
+        ex.rot_mult = s.yarn_factor > 0.f ? 0.1f * std::log(s.yarn_factor) + 1.f : 1.f;
+        for (int i = 0; i < nparts; ++i) {
+            const LmPart&     P = parts[i];
+            GeneralAttnParams p = attn_params(e, L, P);
+            TM_PROF(P_KV_STORE, TM_TRY(launch_attn_prep(src + (size_t)P.row0 * ld, ld, 0, L.c_k, L.c_v, (void*)p.q, lm.ldq, s.qk_norm_w != 0, false,
+                                                        m.norm_eps, p, st, ex)));
+        }
+        TM_TRY(run_attention_parts(e, L, parts, nparts));
+        if (s.diff_maps) {
+            TM_PROF(P_ATTN, TM_TRY(launch_diff_head_norm(lm.d_cat, lm.ldcat, lm.elem, lm.d_mixo, lm.ldmix, L.lambda, 1.f - s.diff_init, M, H, s.vdim,
+                                                         m.norm_eps, st)));
+        }
+        TM_PROF(P_GEMM_O, TM_TRY(launch_dense_linear(L.wo, lm.d_cat, lm.ldcat, lm.d_y, W, M, kDenseScaleF32, 1.f, st)));
+        TM_PROF(P_RES_NORM, TM_TRY(launch_group_rmsnorm_add_f32(lm.d_res, lm.d_h1, lm.ldw, lm.elem, lm.d_y, nullptr, nullptr, nullptr, L.norm1, groups,
+                                                                m.norm_eps, M, W, st)));
+    }
+    else {
+        // ---- left: attention with mixed heads, distance table, zero sink, output gate ----
+        for (int i = 0; i < nparts; ++i) {
+            const LmPart&     P = parts[i];
+            GeneralAttnParams p = attn_params(e, L, P);
+            TM_PROF(P_KV_STORE, TM_TRY(launch_talk_prep(lm.d_proj + (size_t)P.row0 * lm.ldproj, lm.ldproj, 0, L.c_k, (void*)p.q, lm.ldq, L.q_w, L.k_w, L.talk,
+                                                        s.dim, m.norm_eps, p, st)));
+        }
+        TM_TRY(run_attention_parts(e, L, parts, nparts));
+        TM_PROF(P_ATTN, TM_TRY(launch_sigmoid_gate_mul(lm.d_cat, lm.ldcat, lm.elem, lm.d_mixo, lm.ldmix, lm.d_proj + L.c_g, lm.ldproj, M, L.n_att, st)));
+        TM_PROF(P_GEMM_O, TM_TRY(launch_dense_linear(L.wo, lm.d_cat, lm.ldcat, lm.d_y, W, M, kDenseScaleF32, 1.f, st)));
+        // ---- right: gated delta rule ----
+        const int Hr = s.r_heads, dr = s.r_dim, dvr = s.r_vdim;
+        TM_PROF(P_KV_STORE, TM_TRY(launch_act_cast_f32(lm.d_lora, lm.ldlora, lm.elem, lm.d_proj + L.c_a1, lm.ldproj, M, L.lora_g1 + s.g_rank, 0, st)));
+        DenseCall c;
+        c.epi  = kDenseBiasF32;
+        c.bias = L.dt_bias;
+        TM_PROF(P_GEMM_QKV, TM_TRY(launch_dense_call(L.a2, lm.d_lora, lm.ldlora, lm.d_wdec, lm.ldmix, M, c, st)));
+        TM_PROF(P_GEMM_QKV, TM_TRY(launch_dense_linear(L.g2, (const char*)lm.d_lora + (size_t)L.lora_g1 * lm.elem, lm.ldlora, lm.d_gate2, lm.ldmix, M,
+                                                       kDenseScaleF32, 1.f, st)));
+        TM_PROF(P_KV_STORE, TM_TRY(launch_gdelta_prep(lm.d_conv, lm.ldconv, 0, L.r_nqk, L.c_xq, L.c_xk, lm.d_proj + L.c_b, lm.ldproj, lm.d_wdec, lm.ldmix,
+                                                      L.a_log, nullptr, lm.d_aux, lm.ldmix, M, Hr, s.r_kv_heads, dr, st)));
+        for (int i = 0; i < nparts; ++i) {
+            const LmPart&  P  = parts[i];
+            StateMixParams sp = state_seqs(e, P);
+            sp.layer_offset   = L.state_offset;
+            sp.heads = Hr, sp.dim = dr, sp.vdim = dvr;
+            sp.proj = lm.d_conv + (size_t)P.row0 * lm.ldconv, sp.ld = lm.ldconv;
+            sp.c_q = L.c_xq, sp.c_k = L.c_xk, sp.c_a = L.c_xk, sp.c_v = 2 * L.r_nqk;
+            sp.decay_w = lm.d_wdec + (size_t)P.row0 * lm.ldmix, sp.ld_w = lm.ldmix;
+            sp.unit    = lm.d_aux + (size_t)P.row0 * lm.ldmix, sp.ld_u = lm.ldmix;
+            sp.out     = lm.d_mixo + (size_t)P.row0 * lm.ldmix, sp.ldo = lm.ldmix;
+            TM_PROF(P_ATTN, TM_TRY(launch_state_mix(sp, true, st)));
+        }
+        TM_PROF(P_ATTN, TM_TRY(launch_gated_group_norm(lm.d_cat, lm.ldcat, lm.elem, lm.d_mixo, lm.ldmix, L.r_norm, lm.d_gate2, lm.ldmix, M, Hr, dvr,
+                                                       m.norm_eps, st)));
+        TM_PROF(P_GEMM_O, TM_TRY(launch_dense_linear(L.wo_r, lm.d_cat, lm.ldcat, lm.d_y2, W, M, kDenseScaleF32, 1.f, st)));
+        TM_PROF(P_RES_NORM, TM_TRY(launch_group_rmsnorm_add_f32(lm.d_res, lm.d_h1, lm.ldw, lm.elem, lm.d_y, lm.d_y2, L.join_l, L.join_r, L.norm1, groups,
+                                                                m.norm_eps, M, W, st)));
+    }
+    if (s.mlp == TM_MLP_NONE) {
+        return 0;
+    }
+    DenseCall c;  // act(gate) * up leaves the [gate | up] product's epilogue in the activation type
+    c.epi   = kDenseGatedAct;
+    c.act   = s.act;
+    c.n_out = s.ff;
+    TM_PROF(P_GEMM_GATE_UP, TM_TRY(launch_dense_call(L.gu, lm.d_h1, lm.ldw, lm.d_ff, lm.ldff, M, c, st)));
+    TM_PROF(P_GEMM_DOWN, TM_TRY(launch_dense_linear(L.down, lm.d_ff, lm.ldff, lm.d_y, W, M, kDenseScaleF32, 1.f, st)));
+    TM_PROF(P_RES_NORM, TM_TRY(launch_group_rmsnorm_add_f32(lm.d_res, lm.d_h1, lm.ldw, lm.elem, lm.d_y, nullptr, nullptr, nullptr, L.norm2, groups,
+                                                            m.norm_eps, M, W, st)));
+    return 0;
+}
+
 // one post-norm block over M rows (see the head of this file); h_ready: lm.d_h1 already holds the stream in the activation type
 static int post_layer(tm_engine* e, const LmLayer& L, int M, const LmPart* parts, int nparts, bool h_ready)
 {
@@ -803,6 +1156,9 @@ static int post_layer(tm_engine* e, const LmLayer& L, int M, const LmPart* parts
     const int                W = m.width, H = s.heads;
     if (!h_ready) {
         TM_PROF(P_RES_NORM, TM_TRY(launch_act_cast_f32(lm.d_h1, lm.ldw, lm.elem, lm.d_res, W, M, W, 0, st)));
+    }
+    if (s.norm_groups > 0) {
+        return group_layer(e, L, M, parts, nparts);
     }
     DenseCall pc;
     pc.epi  = L.proj_bias ? kDenseBiasF32 : kDenseScaleF32;
@@ -917,7 +1273,7 @@ static int layered_layers(tm_engine* e, const int* d_ids, int M, const LmPart* p
         const LmPart& P = parts[i];
         TM_TRY(launch_rows_prepare(lm.d_row_seq + P.row0, lm.d_row_pos + P.row0, P.cu_q, P.k_len, P.nseq, P.rows, st));
     }
-    TM_PROF(P_EMBED, TM_TRY(launch_embedding_f32(lm.d_res, lm.embed, lm.elem, d_ids, M, m.width, m.vocab, st)));
+    TM_PROF(P_EMBED, TM_TRY(launch_embedding_f32(lm.d_res, lm.embed, lm.elem, d_ids, M, m.width, m.vocab, st, m.embed_scale > 0.f ? m.embed_scale : 1.f)));
     if (m.loop_times > 0) {  // the embedding output is read again where a loop pass begins
         TM_PROF(P_EMBED, TM_TRY(launch_embedding_f32(lm.d_x0, lm.embed, lm.elem, d_ids, M, m.width, m.vocab, st)));
     }
@@ -970,7 +1326,11 @@ static int layered_logits(tm_engine* e, const int* rows, int n)
     LayeredModel&            lm = *e->lm;
     const tm_layered_config& m  = lm.cfg;
     TM_REQUIRE(n <= lm.max_logit_rows, "internal: too many logits rows");
-    if (m.final_layer_norm) {
+    if (m.norm_groups > 0) {
+        TM_PROF(P_RES_NORM, TM_TRY(launch_group_rmsnorm_f32(lm.d_hn, lm.ldw, lm.elem, lm.d_res, rows, lm.final_norm, m.norm_groups, m.norm_eps, n, m.width,
+                                                            e->stream)));
+    }
+    else if (m.final_layer_norm) {
         TM_PROF(P_RES_NORM, TM_TRY(launch_layernorm_f32(lm.d_hn, lm.ldw, lm.elem, lm.d_res, rows, lm.final_norm, lm.final_norm_b, m.norm_eps, n,
                                                         m.width, e->stream)));
     }
@@ -979,6 +1339,9 @@ static int layered_logits(tm_engine* e, const int* rows, int n)
                                                       m.norm_eps, n, m.width, e->stream)));
     }
     TM_PROF(P_LM_HEAD, TM_TRY(launch_dense_linear(lm.head, lm.d_hn, lm.ldw, lm.d_logits_f32, m.vocab, n, kDenseScaleF32, m.logit_scale, e->stream)));
+    if (m.logit_softcap > 0.f) {
+        TM_PROF(P_LM_HEAD, TM_TRY(launch_softcap_f32(lm.d_logits_f32, (size_t)n * m.vocab, m.logit_softcap, e->stream)));
+    }
     return 0;
 }
 
@@ -1037,7 +1400,35 @@ int tm_engine_create_layered(tm_engine** out, const tm_engine_config* c, const t
     for (int i = 0; i < m->n_layers; ++i) {
         const tm_layer_spec& s = m->layers[i];
         const std::string at = "layer " + std::to_string(i);
-        TM_REQUIRE(s.mixer >= TM_MIXER_ATTENTION && s.mixer <= TM_MIXER_DELTA, at + ": unknown mixer");
+        TM_REQUIRE(s.mixer >= TM_MIXER_ATTENTION && s.mixer <= TM_MIXER_PARALLEL, at + ": unknown mixer");
+        TM_REQUIRE(s.post_norm || (s.norm_groups == 0 && s.conv_taps == 0 && !s.diff_maps && !s.rot_pairs && s.yarn_factor == 0.f && s.mixer != TM_MIXER_PARALLEL),
+                   at + ": group norms, convolved projections, differential attention, pairwise rotation and parallel mixers belong to post_norm blocks");
+        if (s.post_norm && s.norm_groups > 0) {
+            TM_REQUIRE(m->width % s.norm_groups == 0 && m->norm_groups > 0, at + ": the width is a multiple of norm_groups; the model's last norm is a group norm too");
+            TM_REQUIRE(s.mixer == TM_MIXER_ATTENTION || s.mixer == TM_MIXER_PARALLEL, at + ": a block with group norms mixes by attention or by the parallel pair");
+            TM_REQUIRE(s.weights_of < 0 && !s.one_norm && !s.resid_gate && s.loop_pass < 0 && !s.sink && !s.dist_bias && !s.out_gate && s.chunk == 0
+                           && !s.qk_unit_norm && !s.v_unit_norm && s.qtemp_coef == 0.f && !s.qkv_bias && s.keep_first == 0,
+                       at + ": a block with group norms takes none of the other block forms' switches");
+            TM_REQUIRE(s.heads >= 1 && s.kv_heads >= 1 && s.heads % s.kv_heads == 0 && s.dim >= 1 && s.dim <= 256 && s.vdim >= 1 && s.vdim <= 256 && s.window >= 0,
+                       at + ": heads % kv_heads, 1 <= dim, vdim <= 256, window >= 0");
+            TM_REQUIRE(s.conv_taps >= 0 && s.conv_taps <= 8, at + ": at most 8 taps");
+            TM_REQUIRE(s.mlp == TM_MLP_NONE || (s.mlp == TM_MLP_GATED && s.ff >= 1 && s.act >= TM_ACT_RELU2 && s.act <= TM_ACT_SILU), at + ": gated feed-forward");
+            if (s.mixer == TM_MIXER_ATTENTION) {
+                TM_REQUIRE(s.rot_dims >= 0 && s.rot_dims % 2 == 0 && s.rot_dims <= s.dim && s.rot_base > 0.f && s.rot_scale > 0.f,
+                           at + ": rot_dims even and <= dim, rot_base, rot_scale > 0");
+                TM_REQUIRE(s.yarn_factor == 0.f || (s.yarn_factor > 0.f && s.yarn_original > 0.f && s.yarn_fast > 0.f && s.yarn_slow > 0.f && s.rot_base != 1.f),
+                           at + ": frequency scaling: factor, original, fast, slow > 0");
+            }
+            else {
+                TM_REQUIRE(s.vdim == s.dim && s.kv_heads * s.dim <= 1024 && s.heads * s.dim <= 12288 && s.dist_buckets >= 2 && s.dist_max > s.dist_buckets / 2
+                               && !s.diff_maps && s.conv_taps == 0 && s.rot_dims == 0 && s.softcap <= 0.f,
+                           at + ": left mixer: vdim = dim, kv_heads * dim <= 1024, dist_buckets >= 2, dist_max > dist_buckets / 2, no maps / convolution / rotation / cap");
+                TM_REQUIRE(s.r_heads >= 1 && s.r_kv_heads >= 1 && s.r_heads % s.r_kv_heads == 0 && s.r_dim >= 1 && s.r_dim <= 256 && s.r_vdim >= 1
+                               && s.r_vdim <= 1024 && s.r_conv >= 1 && s.r_conv <= 8 && s.a_rank >= 1 && s.g_rank >= 1,
+                           at + ": right mixer: r_heads % r_kv_heads, 1 <= r_dim <= 256, 1 <= r_vdim <= 1024, 1 <= r_conv <= 8, a_rank, g_rank >= 1");
+            }
+            continue;
+        }
         TM_REQUIRE(s.post_norm || (s.mixer != TM_MIXER_LIGHTNING && s.mixer != TM_MIXER_DELTA && !s.qkv_bias && !s.qk_norm_w && s.window == 0
                                    && !s.expert_plain && !s.router_softmax && s.shared_ff == 0 && s.act != TM_ACT_XIELU),
                    at + ": state mixers, projection biases, weighted query / key norms, windows, plain experts and xIELU belong to post_norm blocks");
@@ -1049,7 +1440,9 @@ int tm_engine_create_layered(tm_engine** out, const tm_engine_config* c, const t
             TM_REQUIRE(s.weights_of < 0 && !s.one_norm && !s.resid_gate && s.loop_pass < 0 && !s.sink && !s.dist_bias && !s.out_gate && s.chunk == 0
                            && !s.qk_unit_norm && !s.v_unit_norm && s.softcap <= 0.f && s.qtemp_coef == 0.f && s.mixer != TM_MIXER_LATENT,
                        at + ": a post_norm block takes none of the other block forms' switches");
-            TM_REQUIRE(m->final_layer_norm, at + ": post_norm blocks end in a final layer norm");
+            TM_REQUIRE(m->final_layer_norm && m->norm_groups == 0, at + ": post_norm blocks with layer norms end in a final layer norm");
+            TM_REQUIRE(s.mixer != TM_MIXER_PARALLEL && s.conv_taps == 0 && !s.diff_maps && !s.rot_pairs && s.yarn_factor == 0.f,
+                       at + ": the parallel pair, convolved projections, differential attention and pairwise rotation need norm_groups > 0");
             if (s.mixer == TM_MIXER_ATTENTION) {
                 TM_REQUIRE(s.rot_dims >= 0 && s.rot_dims % 2 == 0 && s.rot_dims <= s.dim && s.rot_base > 0.f && s.rot_scale > 0.f,
                            at + ": rot_dims even and <= dim, rot_base, rot_scale > 0");
@@ -1119,13 +1512,93 @@ int tm_engine_create_layered(tm_engine** out, const tm_engine_config* c, const t
         L.n_k      = L.spec.kv_heads * L.spec.dim;
         L.n_v      = L.spec.kv_heads * L.spec.vdim;
         L.n_att    = L.spec.heads * L.spec.vdim;
-        L.a_dim = L.spec.dim, L.a_vdim = L.spec.vdim, L.a_kv = L.spec.kv_heads;
+        L.a_dim = L.spec.dim, L.a_vdim = L.spec.vdim, L.a_kv = L.spec.kv_heads, L.a_heads = L.spec.heads;
         L.post = L.spec.post_norm != 0;
+        L.has_state = L.spec.mixer == TM_MIXER_LIGHTNING || L.spec.mixer == TM_MIXER_DELTA || L.spec.mixer == TM_MIXER_PARALLEL;
+        L.has_cache = L.spec.mixer != TM_MIXER_LIGHTNING && L.spec.mixer != TM_MIXER_DELTA;
         L.wide = !L.post && layer_wide(L.spec);
         auto slot = [&](const std::string& name, int64_t rows, int64_t cols) {
             e->slots[name].bytes = rows * cols * 2;
             lm.fan_in[name]      = (int)cols;
         };
+        if (L.post && L.spec.norm_groups > 0) {
+            const tm_layer_spec& s = L.spec;
+            const int            H = s.heads, G = s.kv_heads, d = s.dim, dv = s.vdim;
+            lm.has_post = true;
+            slot(lname(i, "norm1"), 1, W);
+            if (s.mixer == TM_MIXER_ATTENTION) {
+                const int maps = s.diff_maps ? 2 : 1;
+                L.n_q = H * maps * d, L.n_k = G * maps * d, L.n_v = G * dv, L.n_att = H * dv;
+                L.a_heads = H * maps, L.a_kv = G * maps;
+                if (maps > 1) {  // both maps of a head read the head's one value head
+                    L.a_kh = G * maps, L.a_vh = G;
+                }
+                L.c_k = L.n_q, L.c_v = L.c_k + L.n_k, L.c_g = L.c_end = L.c_v + L.n_v;
+                slot(lname(i, "mix.q"), L.n_q, W);
+                slot(lname(i, "mix.k"), L.n_k, W);
+                slot(lname(i, "mix.v"), L.n_v, W);
+                slot(lname(i, "mix.o"), W, L.n_att);
+                if (s.qk_norm_w) {
+                    slot(lname(i, "mix.q.norm"), 1, d);
+                    slot(lname(i, "mix.k.norm"), 1, d);
+                }
+                if (s.conv_taps > 0) {
+                    L.conv_col = 0, L.conv_ch = L.c_end, L.conv_taps = s.conv_taps, L.conv_act = 0;
+                    slot(lname(i, "mix.q.conv"), L.n_q, s.conv_taps);
+                    slot(lname(i, "mix.k.conv"), L.n_k, s.conv_taps);
+                    slot(lname(i, "mix.v.conv"), L.n_v, s.conv_taps);
+                }
+                if (s.diff_maps) {
+                    for (const char* t : {"mix.lq1", "mix.lk1", "mix.lq2", "mix.lk2"}) {
+                        slot(lname(i, t), 1, d);
+                    }
+                }
+            }
+            else {
+                const int Hr = s.r_heads, Gr = s.r_kv_heads, dr = s.r_dim, dvr = s.r_vdim;
+                // left: one wide key [G dim] shared by all heads (the head mixing lives in the queries), a value head per group
+                L.n_q = H * d, L.n_k = G * d, L.n_v = G * dv, L.n_att = H * dv;
+                L.a_heads = H, L.a_kv = G, L.a_kh = 1, L.a_vh = G, L.a_dim = G * d, L.a_vdim = dv;
+                L.r_nqk = Gr * dr, L.r_nv = Hr * dvr;
+                L.c_k = L.n_q, L.c_g = L.c_k + L.n_k, L.c_rq = L.c_g + L.n_att, L.c_rk = L.c_rq + L.r_nqk, L.c_rv = L.c_rk + L.r_nqk;
+                L.c_b = L.c_rv + L.r_nv, L.c_a1 = L.c_b + Hr, L.lora_g1 = (s.a_rank + 31) / 32 * 32, L.c_g1 = L.c_a1 + L.lora_g1;
+                L.c_end = L.c_g1 + s.g_rank;
+                L.conv_col = L.c_rq, L.conv_ch = 2 * L.r_nqk + L.r_nv, L.conv_taps = s.r_conv, L.conv_act = 1;
+                L.c_xq = L.conv_ch, L.c_xk = L.c_xq + Hr * dr;
+                slot(lname(i, "mix.left.q"), L.n_q, W);
+                slot(lname(i, "mix.left.k"), L.n_k, W);
+                slot(lname(i, "mix.left.q.norm"), 1, L.n_q);
+                slot(lname(i, "mix.left.k.norm"), 1, L.n_k);
+                slot(lname(i, "mix.left.rel"), s.dist_buckets, H);
+                slot(lname(i, "mix.left.talk"), H, H);
+                slot(lname(i, "mix.left.g"), L.n_att, W);
+                slot(lname(i, "mix.left.o"), W, L.n_att);
+                slot(lname(i, "mix.left.out"), 1, W);
+                slot(lname(i, "mix.right.q"), L.r_nqk, W);
+                slot(lname(i, "mix.right.k"), L.r_nqk, W);
+                slot(lname(i, "mix.right.v"), L.r_nv, W);
+                slot(lname(i, "mix.right.q.conv"), L.r_nqk, s.r_conv);
+                slot(lname(i, "mix.right.k.conv"), L.r_nqk, s.r_conv);
+                slot(lname(i, "mix.right.v.conv"), L.r_nv, s.r_conv);
+                slot(lname(i, "mix.right.b"), Hr, W);
+                slot(lname(i, "mix.right.A_log"), 1, Hr);
+                slot(lname(i, "mix.right.norm"), 1, dvr);
+                slot(lname(i, "mix.right.a1"), s.a_rank, W);
+                slot(lname(i, "mix.right.a2"), (int64_t)Hr * dr, s.a_rank);
+                slot(lname(i, "mix.right.dt_bias"), 1, (int64_t)Hr * dr);
+                slot(lname(i, "mix.right.g1"), s.g_rank, W);
+                slot(lname(i, "mix.right.g2"), L.r_nv, s.g_rank);
+                slot(lname(i, "mix.right.o"), W, L.r_nv);
+                slot(lname(i, "mix.right.out"), 1, W);
+            }
+            if (s.mlp) {
+                slot(lname(i, "norm2"), 1, W);
+                slot(lname(i, "mlp.gate"), s.ff, W);
+                slot(lname(i, "mlp.up"), s.ff, W);
+                slot(lname(i, "mlp.down"), W, s.ff);
+            }
+            continue;
+        }
         if (L.post) {
             const tm_layer_spec& s = L.spec;
             const int            H = s.heads;
@@ -1283,7 +1756,7 @@ int tm_engine_create_layered(tm_engine** out, const tm_engine_config* c, const t
     }
     e->slots["embed"].bytes      = W * m->vocab * 2;
     e->slots["final.norm"].bytes = W * 2;
-    if (m->final_layer_norm) {
+    if (m->final_layer_norm && m->norm_groups == 0) {
         e->slots["final.norm.b"].bytes = W * 2;
     }
     e->slots["head"].bytes       = W * m->vocab * 2;

@@ -401,14 +401,17 @@ __global__ __launch_bounds__(256) void attn_prep_kernel(const float* __restrict_
                                                         int ldq, int qk_norm, int v_norm, float eps, GeneralAttnParams p, AttnPrepExtra ex)
 {
     const int lane = threadIdx.x & 63, t = blockIdx.x, u = blockIdx.y * 4 + (threadIdx.x >> 6);
-    const int H = p.q_heads, G = p.kv_heads;
-    if (u >= H + 2 * G) {
+    const int H = p.q_heads, G = p.k_heads > 0 ? p.k_heads : p.kv_heads, GV = p.v_heads > 0 ? p.v_heads : p.kv_heads;
+    if (u >= H + G + GV) {
         return;
     }
-    const int    kind = u < H ? 0 : (u < H + G ? 1 : 2), head = kind == 0 ? u : (kind == 1 ? u - H : u - H - G);
+    const int    kind = u < H ? 0 : (u < H + G ? 1 : 2), src = kind == 0 ? u : (kind == 1 ? u - H : u - H - G);
     const int    n    = kind == 2 ? p.vdim : p.dim;
-    const float* x    = proj + (size_t)t * ld + (kind == 0 ? q_col : (kind == 1 ? k_col : v_col)) + (size_t)head * n;
-    float        inv  = 1.f;
+    const float* x    = proj + (size_t)t * ld + (kind == 0 ? q_col : (kind == 1 ? k_col : v_col)) + (size_t)src * n;
+    // several maps per head leave map-major: source [head][map] -> head map * (heads / maps) + head
+    const int maps = kind == 2 ? 1 : ex.maps, cnt = kind == 0 ? H : G;
+    const int head = maps > 1 ? (src % maps) * (cnt / maps) + src / maps : src;
+    float     inv  = 1.f;
     if (kind == 2 ? v_norm : qk_norm) {
         float ss = 0.f;
         for (int i = lane; i < n; i += 64) {
@@ -417,7 +420,7 @@ __global__ __launch_bounds__(256) void attn_prep_kernel(const float* __restrict_
         inv = 1.0f / sqrtf(group_sum<64>(ss) / (float)n + eps);
     }
     const int s = p.row_seq[t], pos = p.row_pos[t], ti = pos % p.block_len;
-    // queries and keys: norm weight, then the rotation of the first rd channels (channel i pairs with i + rd / 2), all in fp32
+    // queries and keys: norm weight, then the rotation of the first rd channels (channel i pairs with i + rd / 2, or 2i with 2i + 1), all in fp32
     const float* nw = kind == 0 ? ex.q_w : (kind == 1 ? ex.k_w : nullptr);
     const int    rd = kind == 2 ? 0 : ex.rot_dims, half = rd / 2;
     auto         qk = [&](int i) {
@@ -425,11 +428,13 @@ __global__ __launch_bounds__(256) void attn_prep_kernel(const float* __restrict_
         if (i >= rd) {
             return a;
         }
-        const int   o = i < half ? i + half : i - half;
+        const bool  first = ex.rot_pairs ? (i & 1) == 0 : i < half;
+        const int   o = ex.rot_pairs ? (i ^ 1) : (i < half ? i + half : i - half);
         const float b = x[o] * inv * (nw ? nw[o] : 1.f);
         float       sn, cs;
-        sincosf((float)pos * ex.inv_freq[i < half ? i : i - half], &sn, &cs);
-        return i < half ? a * cs - b * sn : a * cs + b * sn;
+        sincosf((float)pos * ex.inv_freq[ex.rot_pairs ? i >> 1 : (i < half ? i : i - half)], &sn, &cs);
+        sn *= ex.rot_mult, cs *= ex.rot_mult;
+        return first ? a * cs - b * sn : a * cs + b * sn;
     };
     if (kind == 0) {
         T* q = q_out + (size_t)t * ldq + (size_t)head * n;
@@ -458,15 +463,90 @@ int launch_attn_prep(const float* proj, int ld, int q_col, int k_col, int v_col,
 {
     TM_REQUIRE(proj && q_out && p.row_seq && p.row_pos && p.block_ptrs && p.block_stride >= 1, "attn_prep: operands");
     TM_REQUIRE(ex.rot_dims >= 0 && ex.rot_dims % 2 == 0 && ex.rot_dims <= p.dim && (ex.rot_dims == 0 || ex.inv_freq), "attn_prep: rotation");
+    const int kh = p.k_heads > 0 ? p.k_heads : p.kv_heads, vh = p.v_heads > 0 ? p.v_heads : p.kv_heads;
+    TM_REQUIRE(ex.maps >= 1 && p.q_heads % ex.maps == 0 && kh % ex.maps == 0, "attn_prep: the maps divide the query and key heads");
     if (p.rows == 0) {
         return 0;
     }
-    const dim3 grid(p.rows, (p.q_heads + 2 * p.kv_heads + 3) / 4);
+    const dim3 grid(p.rows, (p.q_heads + kh + vh + 3) / 4);
     if (p.elem_bytes == 2) {
         attn_prep_kernel<__bf16><<<grid, 256, 0, st>>>(proj, ld, q_col, k_col, v_col, (__bf16*)q_out, ldq, qk_norm, v_norm, eps, p, ex);
     }
     else {
         attn_prep_kernel<float><<<grid, 256, 0, st>>>(proj, ld, q_col, k_col, v_col, (float*)q_out, ldq, qk_norm, v_norm, eps, p, ex);
+    }
+    TM_HIP_CHECK(hipGetLastError());
+    return 0;
+}
+
+// attention with mixed heads as attention over one wide key (see launch_talk_prep): one workgroup per row
+template<class T>
+__global__ __launch_bounds__(256) void talk_prep_kernel(const float* __restrict__ proj, int ld, int q_col, int k_col, T* __restrict__ q_out, int ldq,
+                                                        const float* __restrict__ q_w, const float* __restrict__ k_w,
+                                                        const float* __restrict__ talk, int D, float eps, GeneralAttnParams p)
+{
+    extern __shared__ float tp_lds[];  // the normed queries [H][D]
+    __shared__ float red[4];
+    const int    t = blockIdx.x, H = p.q_heads, G = p.kv_heads, r = H / G, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const float *q = proj + (size_t)t * ld + q_col, *k = proj + (size_t)t * ld + k_col;
+    auto block_sum = [&](float v) {
+        v = group_sum<64>(v);
+        __syncthreads();
+        if (lane == 0) {
+            red[wave] = v;
+        }
+        __syncthreads();
+        return (red[0] + red[1]) + (red[2] + red[3]);
+    };
+    float sq = 0.f, sk = 0.f;
+    for (int i = threadIdx.x; i < H * D; i += 256) {
+        sq = fmaf(q[i], q[i], sq);
+    }
+    for (int i = threadIdx.x; i < G * D; i += 256) {
+        sk = fmaf(k[i], k[i], sk);
+    }
+    const float qinv = 1.0f / sqrtf(block_sum(sq) / (float)(H * D) + eps);
+    const float kinv = 1.0f / sqrtf(block_sum(sk) / (float)(G * D) + eps);
+    for (int i = threadIdx.x; i < H * D; i += 256) {
+        tp_lds[i] = q[i] * qinv * q_w[i];
+    }
+    __syncthreads();
+    // Q'[h][c D + d] = sum over the heads g of group c of talk[h][g] q_g[d]
+    for (int i = threadIdx.x; i < H * G * D; i += 256) {
+        const int h = i / (G * D), c = (i / D) % G, d = i % D;
+        float     acc = 0.f;
+        for (int g = c * r; g < (c + 1) * r; ++g) {
+            acc = fmaf(talk[h * H + g], tp_lds[g * D + d], acc);
+        }
+        q_out[(size_t)t * ldq + i] = (T)acc;
+    }
+    const int s = p.row_seq[t], pos = p.row_pos[t], ti = pos % p.block_len;
+    char*     base = (char*)p.block_ptrs[(size_t)(p.seq_slot ? p.seq_slot[s] : s) * p.block_stride + pos / p.block_len] + p.layer_offset;
+    T*        kc   = (T*)base + (size_t)ti * (G * D);   // one key head of size G D
+    T*        vc   = (T*)(base + p.v_offset) + ti;      // G value heads [D][block_len]: channel c D + d of the row at (c D + d) * block_len
+    for (int i = threadIdx.x; i < G * D; i += 256) {
+        kc[i]                         = (T)(k[i] * kinv * k_w[i]);
+        vc[(size_t)i * p.block_len] = (T)k[i];
+    }
+}
+
+int launch_talk_prep(const float* proj, int ld, int q_col, int k_col, void* q_out, int ldq, const float* q_w, const float* k_w, const float* talk,
+                     int head_dim, float eps, const GeneralAttnParams& p, hipStream_t st)
+{
+    TM_REQUIRE(proj && q_out && q_w && k_w && talk && p.row_seq && p.row_pos && p.block_ptrs && p.block_stride >= 1, "talk_prep: operands");
+    TM_REQUIRE(head_dim >= 1 && p.kv_heads >= 1 && p.q_heads % p.kv_heads == 0 && p.k_heads == 1 && p.v_heads == p.kv_heads
+                   && p.dim == p.kv_heads * head_dim && p.vdim == head_dim && ldq >= p.q_heads * p.dim,
+               "talk_prep: one key head of kv_heads * head_dim channels, kv_heads value heads of head_dim");
+    TM_REQUIRE((size_t)p.q_heads * head_dim * 4 <= 48 * 1024, "talk_prep: heads * dim <= 12288");
+    if (p.rows == 0) {
+        return 0;
+    }
+    const size_t lds = (size_t)p.q_heads * head_dim * 4;
+    if (p.elem_bytes == 2) {
+        talk_prep_kernel<__bf16><<<p.rows, 256, lds, st>>>(proj, ld, q_col, k_col, (__bf16*)q_out, ldq, q_w, k_w, talk, head_dim, eps, p);
+    }
+    else {
+        talk_prep_kernel<float><<<p.rows, 256, lds, st>>>(proj, ld, q_col, k_col, (float*)q_out, ldq, q_w, k_w, talk, head_dim, eps, p);
     }
     TM_HIP_CHECK(hipGetLastError());
     return 0;

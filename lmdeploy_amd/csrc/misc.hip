@@ -292,18 +292,19 @@ int ensure_dynamic_lds(const void* kernel, int bytes)
 
 
 template<class T>
-__global__ void embedding_f32_kernel(float* __restrict__ out, const T* __restrict__ table, const int* __restrict__ ids, int T_, int H, int vocab)
+__global__ void embedding_f32_kernel(float* __restrict__ out, const T* __restrict__ table, const int* __restrict__ ids, int T_, int H, int vocab,
+                                     float scale)
 {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i < (size_t)T_ * H) {
         const int t = (int)(i / H), c = (int)(i % H);
         int       id = ids[t];
         id           = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
-        out[i]       = (float)table[(size_t)id * H + c];
+        out[i]       = (float)table[(size_t)id * H + c] * scale;
     }
 }
 
-int launch_embedding_f32(float* out, const void* table, int table_elem_bytes, const int* ids, int T, int H, int vocab, hipStream_t st)
+int launch_embedding_f32(float* out, const void* table, int table_elem_bytes, const int* ids, int T, int H, int vocab, hipStream_t st, float scale)
 {
     TM_REQUIRE(out && table && ids && (table_elem_bytes == 2 || table_elem_bytes == 4), "embedding_f32: operands");
     const size_t n = (size_t)T * H;
@@ -311,10 +312,10 @@ int launch_embedding_f32(float* out, const void* table, int table_elem_bytes, co
         return 0;
     }
     if (table_elem_bytes == 2) {
-        embedding_f32_kernel<__bf16><<<(n + 255) / 256, 256, 0, st>>>(out, (const __bf16*)table, ids, T, H, vocab);
+        embedding_f32_kernel<__bf16><<<(n + 255) / 256, 256, 0, st>>>(out, (const __bf16*)table, ids, T, H, vocab, scale);
     }
     else {
-        embedding_f32_kernel<float><<<(n + 255) / 256, 256, 0, st>>>(out, (const float*)table, ids, T, H, vocab);
+        embedding_f32_kernel<float><<<(n + 255) / 256, 256, 0, st>>>(out, (const float*)table, ids, T, H, vocab, scale);
     }
     TM_HIP_CHECK(hipGetLastError());
     return 0;
@@ -368,6 +369,94 @@ int launch_concat2(void* out, int ldo, int out_elem_bytes, const float* a, const
         concat2_kernel<float><<<(total + 255) / 256, 256, 0, st>>>((float*)out, ldo, a, b, H, total);
     }
     TM_HIP_CHECK(hipGetLastError());
+    return 0;
+}
+
+// ---- mixer outputs on their way to the output projection ------------------------------------------------------------------------------
+// differential attention: one wave per (row, head) joins the head's two maps, o = a1 - lambda a2, and scales o to unit RMS (times mult)
+template<class T>
+__global__ __launch_bounds__(256) void diff_head_norm_kernel(T* __restrict__ y, int ldy, const float* __restrict__ a, int lda,
+                                                             const float* __restrict__ lambda, float mult, int heads, int n, float eps)
+{
+    const int t = blockIdx.x, h = blockIdx.y * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+    if (h >= heads) {
+        return;
+    }
+    const float  lam = lambda[0];
+    const float *a1 = a + (size_t)t * lda + (size_t)h * n, *a2 = a1 + (size_t)heads * n;
+    float        ss = 0.f;
+    for (int i = lane; i < n; i += 64) {
+        const float o = fmaf(-lam, a2[i], a1[i]);
+        ss            = fmaf(o, o, ss);
+    }
+    const float inv = mult / sqrtf(group_sum<64>(ss) / (float)n + eps);
+    for (int i = lane; i < n; i += 64) {
+        y[(size_t)t * ldy + (size_t)h * n + i] = (T)(fmaf(-lam, a2[i], a1[i]) * inv);
+    }
+}
+
+int launch_diff_head_norm(void* y, int ldy, int out_elem_bytes, const float* a, int lda, const float* lambda, float mult, int rows, int heads, int n,
+                          float eps, hipStream_t st)
+{
+    TM_REQUIRE(y && a && lambda && heads >= 1 && n >= 1 && ldy >= heads * n && lda >= 2 * heads * n && (out_elem_bytes == 2 || out_elem_bytes == 4),
+               "diff_head_norm: operands");
+    if (rows == 0) {
+        return 0;
+    }
+    const dim3 grid(rows, (heads + 3) / 4);
+    if (out_elem_bytes == 2) {
+        diff_head_norm_kernel<__bf16><<<grid, 256, 0, st>>>((__bf16*)y, ldy, a, lda, lambda, mult, heads, n, eps);
+    }
+    else {
+        diff_head_norm_kernel<float><<<grid, 256, 0, st>>>((float*)y, ldy, a, lda, lambda, mult, heads, n, eps);
+    }
+    TM_HIP_CHECK(hipGetLastError());
+    return 0;
+}
+
+template<class T>
+__global__ void sigmoid_gate_mul_kernel(T* __restrict__ y, int ldy, const float* __restrict__ x, int ldx, const float* __restrict__ gate, int ldg,
+                                        int rows, int n)
+{
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < (size_t)rows * n) {
+        const int t = (int)(i / n), c = (int)(i % n);
+        y[(size_t)t * ldy + c] = (T)(x[(size_t)t * ldx + c] / (1.f + expf(-gate[(size_t)t * ldg + c])));
+    }
+}
+
+int launch_sigmoid_gate_mul(void* y, int ldy, int out_elem_bytes, const float* x, int ldx, const float* gate, int ldg, int rows, int n, hipStream_t st)
+{
+    TM_REQUIRE(y && x && gate && n >= 1 && ldy >= n && ldx >= n && ldg >= n && (out_elem_bytes == 2 || out_elem_bytes == 4), "sigmoid_gate_mul: operands");
+    const size_t total = (size_t)rows * n;
+    if (total == 0) {
+        return 0;
+    }
+    if (out_elem_bytes == 2) {
+        sigmoid_gate_mul_kernel<__bf16><<<(total + 255) / 256, 256, 0, st>>>((__bf16*)y, ldy, x, ldx, gate, ldg, rows, n);
+    }
+    else {
+        sigmoid_gate_mul_kernel<float><<<(total + 255) / 256, 256, 0, st>>>((float*)y, ldy, x, ldx, gate, ldg, rows, n);
+    }
+    TM_HIP_CHECK(hipGetLastError());
+    return 0;
+}
+
+__global__ void softcap_f32_kernel(float* __restrict__ x, size_t n, float cap)
+{
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) {
+        x[i] = cap * tanhf(x[i] / cap);
+    }
+}
+
+int launch_softcap_f32(float* x, size_t n, float cap, hipStream_t st)
+{
+    TM_REQUIRE(x && cap > 0.f, "softcap_f32: operands");
+    if (n > 0) {
+        softcap_f32_kernel<<<(n + 255) / 256, 256, 0, st>>>(x, n, cap);
+        TM_HIP_CHECK(hipGetLastError());
+    }
     return 0;
 }
 

@@ -284,6 +284,101 @@ int launch_layernorm_add_f32(float* x, void* h, int ldh, int h_elem_bytes, const
     return 0;
 }
 
+// RMS norm in groups, one workgroup per row; the row is staged in LDS (H + groups floats), wave w reduces the groups w, w + 4, ...
+// JOIN: the normed vector is 0.5 (r / rms(r) jw + r2 / rms(r2) jw2), each RMS over the whole row.  ADD: x[m] += GN(.), the new row is
+// also written in the activation type
+template<class T, bool ADD>
+__global__ __launch_bounds__(256) void group_rmsnorm_f32_kernel(T* __restrict__ y, int ldy, float* __restrict__ xs, const float* __restrict__ src,
+                                                                const float* __restrict__ src2, const float* __restrict__ jw,
+                                                                const float* __restrict__ jw2, const int* __restrict__ rows,
+                                                                const float* __restrict__ w, int groups, float eps, int H)
+{
+    extern __shared__ float gn_lds[];
+    __shared__ float red[4];
+    float*       row = gn_lds;
+    float*       inv = gn_lds + H;
+    const int    m = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const size_t r0 = (size_t)(rows ? rows[m] : m) * H;
+    if (src2) {
+        float s1 = 0.f, s2 = 0.f;
+        for (int i = threadIdx.x; i < H; i += 256) {
+            const float a = src[r0 + i], b = src2[r0 + i];
+            s1 = fmaf(a, a, s1);
+            s2 = fmaf(b, b, s2);
+        }
+        const float i1 = 1.0f / sqrtf(block_sum_256(s1, red) / (float)H + eps);
+        const float i2 = 1.0f / sqrtf(block_sum_256(s2, red) / (float)H + eps);
+        for (int i = threadIdx.x; i < H; i += 256) {
+            row[i] = 0.5f * (src[r0 + i] * i1 * jw[i] + src2[r0 + i] * i2 * jw2[i]);
+        }
+    }
+    else {
+        for (int i = threadIdx.x; i < H; i += 256) {
+            row[i] = src[r0 + i];
+        }
+    }
+    __syncthreads();
+    const int n = H / groups;
+    for (int g = wave; g < groups; g += 4) {
+        float ss = 0.f;
+        for (int i = lane; i < n; i += 64) {
+            const float v = row[g * n + i];
+            ss            = fmaf(v, v, ss);
+        }
+        ss = group_sum<64>(ss);
+        if (lane == 0) {
+            inv[g] = 1.0f / sqrtf(ss / (float)n + eps);
+        }
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < H; i += 256) {
+        float o = row[i] * inv[i / n] * w[i];
+        if constexpr (ADD) {
+            o += xs[(size_t)m * H + i];
+            xs[(size_t)m * H + i] = o;
+        }
+        y[(size_t)m * ldy + i] = (T)o;
+    }
+}
+
+int launch_group_rmsnorm_f32(void* y, int ldy, int out_elem_bytes, const float* x, const int* rows, const float* w, int groups, float eps, int M,
+                             int H, hipStream_t st)
+{
+    TM_REQUIRE(y && x && w && ldy >= H && (out_elem_bytes == 2 || out_elem_bytes == 4), "group_rmsnorm_f32: operands");
+    TM_REQUIRE(groups >= 1 && H % groups == 0 && H + groups <= 16000, "group_rmsnorm_f32: the width is a multiple of the groups, at most 16000 floats in LDS");
+    if (M == 0) {
+        return 0;
+    }
+    const size_t lds = (size_t)(H + groups) * 4;
+    if (out_elem_bytes == 2) {
+        group_rmsnorm_f32_kernel<__bf16, false><<<M, 256, lds, st>>>((__bf16*)y, ldy, nullptr, x, nullptr, nullptr, nullptr, rows, w, groups, eps, H);
+    }
+    else {
+        group_rmsnorm_f32_kernel<float, false><<<M, 256, lds, st>>>((float*)y, ldy, nullptr, x, nullptr, nullptr, nullptr, rows, w, groups, eps, H);
+    }
+    TM_HIP_CHECK(hipGetLastError());
+    return 0;
+}
+
+int launch_group_rmsnorm_add_f32(float* x, void* h, int ldh, int h_elem_bytes, const float* r, const float* r2, const float* jw, const float* jw2,
+                                 const float* w, int groups, float eps, int M, int H, hipStream_t st)
+{
+    TM_REQUIRE(x && h && r && w && ldh >= H && (h_elem_bytes == 2 || h_elem_bytes == 4) && (!r2 || (jw && jw2)), "group_rmsnorm_add_f32: operands");
+    TM_REQUIRE(groups >= 1 && H % groups == 0 && H + groups <= 16000, "group_rmsnorm_add_f32: the width is a multiple of the groups, at most 16000 floats in LDS");
+    if (M == 0) {
+        return 0;
+    }
+    const size_t lds = (size_t)(H + groups) * 4;
+    if (h_elem_bytes == 2) {
+        group_rmsnorm_f32_kernel<__bf16, true><<<M, 256, lds, st>>>((__bf16*)h, ldh, x, r, r2, jw, jw2, nullptr, w, groups, eps, H);
+    }
+    else {
+        group_rmsnorm_f32_kernel<float, true><<<M, 256, lds, st>>>((float*)h, ldh, x, r, r2, jw, jw2, nullptr, w, groups, eps, H);
+    }
+    TM_HIP_CHECK(hipGetLastError());
+    return 0;
+}
+
 // y = act(x) in the activation type: the stream as a GEMM operand (act 0), tanh of a low-rank projection (act 1)
 template<class T>
 __global__ void act_cast_f32_kernel(T* __restrict__ y, int ldy, const float* __restrict__ x, int ldx, int M, int H, int act)

@@ -3,6 +3,9 @@
 //   linear attention ("lightning"):  S <- decay[head] S + k v^T                         o = S^T q      q, k, v = silu(projection)
 //   generalized delta rule:          S <- diag(w) S - (a u)(u^T S) + k v^T              o = S^T r      u = k / sqrt(|k|^2 + 1e-6),
 //                                    w, a per key channel (both terms read the old S)
+//   gated delta rule:                S <- diag(g) S;  S <- S + k (beta (v - S^T k))^T   o = S^T q      is the same recurrence with
+//                                    w = g, u = g k, a u = beta k and the key beta k (launch_gdelta_prep forms these vectors)
+//   short convolution:               y_t = sum_j w[:, j] u_(t - taps + 1 + j) per channel; its state is the last taps - 1 inputs
 //
 // State pool: one state per (slot, layer run) -- slot = the engine's batch slot of the sequence, plus one parking slot for the decode
 // rows of slots that hold no running sequence.  A sequence whose first row of a launch has position 0 starts from zero whatever the
@@ -388,7 +391,7 @@ int launch_state_mix(const StateMixParams& p, bool delta, hipStream_t st)
 {
     TM_REQUIRE(p.nseq >= 0 && p.heads >= 1 && p.dim >= 1 && p.dim <= 256 && p.vdim >= 1 && p.max_q_len >= 1, "state mixer: sizes (dim <= 256)");
     TM_REQUIRE(p.cu_q && p.k_len && p.state && p.proj && p.out && p.ld >= 1 && p.ldo >= p.heads * p.vdim, "state mixer: operands");
-    TM_REQUIRE(delta ? (p.decay_w && p.unit && p.ld_w >= p.heads * p.dim && p.ld_u >= p.heads * p.dim && p.vdim == p.dim) : p.decay_h != nullptr,
+    TM_REQUIRE(delta ? (p.decay_w && p.unit && p.ld_w >= p.heads * p.dim && p.ld_u >= p.heads * p.dim) : p.decay_h != nullptr,
                "state mixer: decay operands");
     if (p.nseq == 0) {
         return 0;
@@ -441,6 +444,138 @@ int launch_delta_prep(float* proj, int ld, int c_k, int c_a, float* decay, int l
         return 0;
     }
     delta_prep_kernel<<<dim3(rows, (heads + 3) / 4), 256, 0, st>>>(proj, ld, c_k, c_a, decay, ld_w, unit, ld_u, heads, dim);
+    TM_HIP_CHECK(hipGetLastError());
+    return 0;
+}
+
+// gated delta rule: one wave per (row, head) turns the convolved queries / keys and the decay logits into the vectors of the recurrence
+__global__ __launch_bounds__(256) void gdelta_prep_kernel(float* __restrict__ src, int ld, int c_q, int c_k, int c_qo, int c_ko,
+                                                          const float* __restrict__ beta_logit, int ld_b, float* __restrict__ decay, int ld_w,
+                                                          const float* __restrict__ a_log, const float* __restrict__ dt_bias,
+                                                          float* __restrict__ unit, int ld_u, int H, int G, int D)
+{
+    const int t = blockIdx.x, h = blockIdx.y * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+    if (h >= H) {
+        return;
+    }
+    const int    c  = h / (H / G);
+    float*       pr = src + (size_t)t * ld;
+    const float *q = pr + c_q + c * D, *k = pr + c_k + c * D;
+    float        sq = 0.f, sk = 0.f;
+    for (int i = lane; i < D; i += 64) {
+        sq = fmaf(q[i], q[i], sq);
+        sk = fmaf(k[i], k[i], sk);
+    }
+    const float qinv = 1.0f / (sqrtf(group_sum<64>(sq) + 1e-6f) * sqrtf((float)D));
+    const float kinv = 1.0f / sqrtf(group_sum<64>(sk) + 1e-6f);
+    const float beta = 1.f / (1.f + expf(-beta_logit[(size_t)t * ld_b + h]));
+    const float A    = expf(a_log[h]);
+    for (int i = lane; i < D; i += 64) {
+        const float ku = k[i] * kinv;
+        float&      w  = decay[(size_t)t * ld_w + h * D + i];
+        const float z  = w + (dt_bias ? dt_bias[h * D + i] : 0.f);
+        const float g  = expf(-A * (z > 20.f ? z : log1pf(expf(z))));
+        w                                  = g;
+        pr[c_qo + h * D + i]               = q[i] * qinv;
+        pr[c_ko + h * D + i]               = beta * ku;
+        unit[(size_t)t * ld_u + h * D + i] = g * ku;
+    }
+}
+
+int launch_gdelta_prep(float* src, int ld, int c_q, int c_k, int c_qo, int c_ko, const float* beta_logit, int ld_b, float* decay, int ld_w,
+                       const float* a_log, const float* dt_bias, float* unit, int ld_u, int rows, int heads, int kv_heads, int dim, hipStream_t st)
+{
+    TM_REQUIRE(src && beta_logit && decay && a_log && unit && heads >= 1 && kv_heads >= 1 && heads % kv_heads == 0 && dim >= 1, "gdelta prep: operands");
+    TM_REQUIRE(c_qo >= c_q + kv_heads * dim && c_qo >= c_k + kv_heads * dim && c_ko >= c_qo + heads * dim && ld >= c_ko + heads * dim,
+               "gdelta prep: the per-head vectors lie behind the convolved ones");
+    if (rows == 0) {
+        return 0;
+    }
+    gdelta_prep_kernel<<<dim3(rows, (heads + 3) / 4), 256, 0, st>>>(src, ld, c_q, c_k, c_qo, c_ko, beta_logit, ld_b, decay, ld_w, a_log, dt_bias, unit,
+                                                                    ld_u, heads, kv_heads, dim);
+    TM_HIP_CHECK(hipGetLastError());
+    return 0;
+}
+
+// short causal convolution: thread = (sequence, channel, segment of kConvSeg rows); it keeps the last taps - 1 inputs in registers, so every
+// input is read once.  A segment's first rows read the rows before it from x (x is not written: the output goes elsewhere) or, before the
+// launch's first row, from the sequence's state; the thread of segment 0 then stores the state's new content -- nobody else touches it.
+// MT: register window, taps <= MT; weights are right-aligned in it (unused taps weigh zero)
+constexpr int kConvSeg = 64;
+
+template<int MT>
+__global__ __launch_bounds__(256) void short_conv_kernel(float* __restrict__ y, int ldy, const float* __restrict__ x, int ldx, int x_col,
+                                                         const float* __restrict__ w, int C, int taps, int act, StateMixParams p)
+{
+    const int s = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x, seg = blockIdx.z;
+    const int row0 = p.cu_q[s] - p.cu_q[0], q_len = p.cu_q[s + 1] - p.cu_q[s];
+    const int t0 = seg * kConvSeg, t1 = min(q_len, t0 + kConvSeg);
+    if (c >= C || (t0 >= q_len && seg > 0)) {
+        return;
+    }
+    const int pos0 = p.k_len[s] - q_len, nh = taps - 1;
+    int       slot = p.seq_slot ? p.seq_slot[s] : p.slot0 + s;
+    if (p.active && !p.active[s]) {
+        slot = p.park_slot;
+    }
+    float* st = p.state + (size_t)slot * p.slot_stride + p.layer_offset;  // [taps - 1][C]
+    // input at row t of the launch's rows of this sequence (t < 0: history)
+    auto input = [&](int t) -> float {
+        if (t >= 0) {
+            return x[(size_t)(row0 + t) * ldx + x_col + c];
+        }
+        return (pos0 > 0 && t + nh >= 0) ? st[(size_t)(t + nh) * C + c] : 0.f;
+    };
+    float wt[MT], win[MT - 1];
+#pragma unroll
+    for (int k = 0; k < MT; ++k) {
+        const int j = k - (MT - taps);  // tap index
+        wt[k]       = j >= 0 ? w[(size_t)c * taps + j] : 0.f;
+    }
+#pragma unroll
+    for (int k = 0; k < MT - 1; ++k) {
+        const int j = k - (MT - 1 - nh);  // history index 0 .. nh - 1, oldest first
+        win[k]      = j >= 0 ? input(t0 - nh + j) : 0.f;
+    }
+    for (int t = t0; t < t1; ++t) {
+        const float u   = x[(size_t)(row0 + t) * ldx + x_col + c];
+        float       acc = 0.f;
+#pragma unroll
+        for (int k = 0; k < MT - 1; ++k) {
+            acc = fmaf(wt[k], win[k], acc);
+        }
+        acc = fmaf(wt[MT - 1], u, acc);
+#pragma unroll
+        for (int k = 0; k + 1 < MT - 1; ++k) {
+            win[k] = win[k + 1];
+        }
+        if (MT > 1) {
+            win[MT - 2] = u;
+        }
+        y[(size_t)(row0 + t) * ldy + c] = act == 1 ? sm_silu(acc) : acc;
+    }
+    if (seg == 0) {  // new state: the inputs q_len - nh .. q_len - 1; ascending j reads st behind what it has written
+        for (int j = 0; j < nh; ++j) {
+            st[(size_t)j * C + c] = input(q_len - nh + j);
+        }
+    }
+}
+
+int launch_short_conv(float* y, int ldy, const float* x, int ldx, int x_col, const float* w, int channels, int taps, int act,
+                      const StateMixParams& p, hipStream_t st)
+{
+    TM_REQUIRE(y && x && w && channels >= 1 && ldy >= channels && ldx >= x_col + channels && taps >= 1 && taps <= 8, "short conv: operands (1 <= taps <= 8)");
+    TM_REQUIRE(p.cu_q && p.k_len && (taps == 1 || p.state) && p.max_q_len >= 1, "short conv: sequences / state");
+    if (p.nseq == 0) {
+        return 0;
+    }
+    const dim3 grid(p.nseq, (channels + 255) / 256, (p.max_q_len + kConvSeg - 1) / kConvSeg);
+    if (taps <= 4) {
+        short_conv_kernel<4><<<grid, 256, 0, st>>>(y, ldy, x, ldx, x_col, w, channels, taps, act, p);
+    }
+    else {
+        short_conv_kernel<8><<<grid, 256, 0, st>>>(y, ldy, x, ldx, x_col, w, channels, taps, act, p);
+    }
     TM_HIP_CHECK(hipGetLastError());
     return 0;
 }

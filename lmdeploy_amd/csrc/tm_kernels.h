@@ -424,6 +424,14 @@ struct GeneralAttnParams {
     const float*    out_gate = nullptr;  // [rows][ld_gate] or nullptr: head h of row t is multiplied by sigmoid(out_gate[t][h])
     int             ld_gate = 0;
     int             out_head_stride = 0; // > 0: head h of an output row starts at h * out_head_stride instead of h * vdim
+    // the query heads form kv_heads groups of q_heads / kv_heads consecutive heads; group g reads key head g % k_heads and value head
+    // g % v_heads of a cache that holds keys [k_heads][block_len][dim] and values [v_heads][vdim][block_len] (0: kv_heads of each).
+    // Two score maps over the same values: 2 G key heads, G value heads.  One wide key shared by every group with a value head per
+    // group: 1 key head, G value heads.
+    int             k_heads = 0, v_heads = 0;
+    const float*    dist_table = nullptr;  // [q_heads][dist_table_len] or nullptr: score += dist_table[head][min(position - key position, len - 1)]
+    int             dist_table_len = 0;
+    int             out_f32 = 0;           // != 0: the output rows are fp32 whatever the cache's element type
     int             splits = 1;
     float*          partial_o = nullptr;   // [rows][q_heads][splits][vdim]
     float*          partial_ml = nullptr;  // [rows][q_heads][splits][2]
@@ -449,8 +457,8 @@ int    launch_general_attention(const GeneralAttnParams& p, bool prefill, hipStr
 // parallel block share one statistic.  x fp32 [.][H]; y bf16 | fp32 [M][ldy]; w fp32 [H]
 int launch_rmsnorm_f32(void* y0, void* y1, int ldy, int out_elem_bytes, const float* x, const int* rows, const float* w0, const float* w1,
                        float w_offset, float eps, int M, int H, hipStream_t st);
-// out fp32 [T][H] = table[ids[t]] (table bf16 | fp32 [vocab][H])
-int launch_embedding_f32(float* out, const void* table, int table_elem_bytes, const int* ids, int T, int H, int vocab, hipStream_t st);
+// out fp32 [T][H] = table[ids[t]] * scale (table bf16 | fp32 [vocab][H])
+int launch_embedding_f32(float* out, const void* table, int table_elem_bytes, const int* ids, int T, int H, int vocab, hipStream_t st, float scale = 1.f);
 // row_seq / row_pos of the rows [0, cu_q[nseq]) of nseq sequences: position = k_len[s] - (cu_q[s + 1] - cu_q[s]) + offset in the sequence
 int launch_rows_prepare(int* row_seq, int* row_pos, const int* cu_q, const int* k_len, int nseq, int rows, hipStream_t st);
 // keys / values of the new rows -> paged cache.  qkv [rows][ld]: keys at column k_col ([kv_heads][dim]), values at v_col ([kv_heads][vdim])
@@ -459,12 +467,25 @@ int launch_kv_store_general(const void* qkv, int ld, int k_col, int v_col, const
 // queries -> q_out [rows][ldq] in the cache's element type
 // q_w / k_w (fp32 [dim], may be nullptr): weights of the query / key norm; rot_dims > 0: after the norm the first rot_dims channels of every
 // query and key head turn, channel i with i + rot_dims / 2, by the angle position * inv_freq[i] (fp32)
+// maps = 2: the source holds [map 1 | map 2] per query / key head; the maps leave as heads of their own, map-major (source head h, map
+// m -> head m * heads / 2 + h), so that a group of query heads and its key head belong to one map.  rot_pairs: channel 2i turns with
+// 2i + 1 instead of i with i + rot_dims / 2.  rot_mult multiplies cos and sin.
 struct AttnPrepExtra {
     const float *q_w = nullptr, *k_w = nullptr, *inv_freq = nullptr;
     int          rot_dims = 0;
+    int          maps = 1, rot_pairs = 0;
+    float        rot_mult = 1.f;
 };
 int launch_attn_prep(const float* proj, int ld, int q_col, int k_col, int v_col, void* q_out, int ldq, bool qk_norm, bool v_norm, float eps,
                      const GeneralAttnParams& layout, hipStream_t st, AttnPrepExtra extra = AttnPrepExtra());
+// attention whose heads' scores are mixed by a matrix T [heads][heads] before the soft-max, as attention over ONE wide key: with
+// s'_h = sum_g T[h][g] scale (q_g . k_kv(g)) the mixed query of head h is Q'_h = [sum_(g in group c) T[h][g] q_g]_(c = 0 .. G-1) (size G dim)
+// against the key [k_0 | ... | k_(G-1)].  proj [rows][ld] fp32: queries ([H][dim]) at q_col, keys ([G][dim]) at k_col; both are RMS-normed over
+// their whole row part with weights q_w / k_w.  Mixed queries -> q_out [rows][ldq] (head h at h * G * dim); normed keys -> the cache's one
+// key head; the keys AS PROJECTED -> the cache's G value heads (value size = dim).  layout: q_heads = H, kv_heads = v_heads = G, k_heads = 1,
+// dim = G * dim
+int launch_talk_prep(const float* proj, int ld, int q_col, int k_col, void* q_out, int ldq, const float* q_w, const float* k_w, const float* talk,
+                     int head_dim, float eps, const GeneralAttnParams& layout, hipStream_t st);
 // latent attention (layout: one key head, dim = C + R, vdim = C): normed latent vector + rotated shared key part -> cache; unrotated query
 // parts -> q_plain (head h at h * plain_stride), rotated query parts -> q_full[h * (C + R) + C ...]
 int launch_latent_prep(const float* proj, int ld, int q_col, int dkv_col, void* q_plain, int ldp, int plain_stride, void* q_full, int ldq,
@@ -490,6 +511,14 @@ int launch_layernorm_f32(void* y, int ldy, int out_elem_bytes, const float* x, c
                          int H, hipStream_t st);
 int launch_layernorm_add_f32(float* x, void* h, int ldh, int h_elem_bytes, const float* r, const float* w, const float* b, float eps, int M, int H,
                              hipStream_t st);
+// RMS norm in groups on the fp32 stream: the row is split into `groups` equal consecutive parts, each divided by its own
+// sqrt(mean(part^2) + eps), the whole times w.  launch_group_rmsnorm_f32: y[m] = GN(x[rows ? rows[m] : m]);
+// launch_group_rmsnorm_add_f32: x[m] += GN(r[m]) and the updated row also goes to h in the activation type.  r2 != nullptr: the normed
+// vector is first 0.5 * (r / rms(r) * jw + r2 / rms(r2) * jw2) (two branches joined, RMS over the whole row)
+int launch_group_rmsnorm_f32(void* y, int ldy, int out_elem_bytes, const float* x, const int* rows, const float* w, int groups, float eps, int M,
+                             int H, hipStream_t st);
+int launch_group_rmsnorm_add_f32(float* x, void* h, int ldh, int h_elem_bytes, const float* r, const float* r2, const float* jw, const float* jw2,
+                                 const float* w, int groups, float eps, int M, int H, hipStream_t st);
 // y [M][ldy] (bf16 | fp32) = act(x [M][ldx] fp32), act: 0 none, 1 tanh
 int launch_act_cast_f32(void* y, int ldy, int out_elem_bytes, const float* x, int ldx, int M, int H, int act, hipStream_t st);
 
@@ -518,8 +547,28 @@ size_t state_mix_floats(int heads, int dim, int vdim);  // floats of one layer's
 int    launch_state_mix(const StateMixParams& p, bool delta, hipStream_t st);
 int    launch_delta_prep(float* proj, int ld, int c_k, int c_a, float* decay, int ld_w, float* unit, int ld_u, int rows, int heads, int dim,
                          hipStream_t st);
+// gated delta rule, per (row, head): what launch_state_mix(delta) reads.  src [rows][ld]: convolved + silu'd queries at c_q and keys at c_k
+// ([kv_heads][dim]); head h uses q / k head h / (heads / kv_heads).  Written: src[.. c_qo + h dim ..] = q / sqrt(|q|^2 + 1e-6) / sqrt(dim);
+// src[.. c_ko + h dim ..] = beta k^ (k^ the unit key, beta = sigmoid(beta_logit[row][h])); decay[row][h dim ..] <- g = exp(-exp(a_log[h])
+// softplus(decay + dt_bias)) in place; unit[row][h dim ..] = g k^
+int    launch_gdelta_prep(float* src, int ld, int c_q, int c_k, int c_qo, int c_ko, const float* beta_logit, int ld_b, float* decay, int ld_w,
+                          const float* a_log, const float* dt_bias, float* unit, int ld_u, int rows, int heads, int kv_heads, int dim, hipStream_t st);
+// short causal convolution over time with its state: y[t][c] = act(sum_j w[c][j] u[t - taps + 1 + j][c]), c < channels, u = x[.][x_col + c]
+// (fp32 [rows][ldx]); rows before the launch's first row of a sequence come from the sequence's state [taps - 1][channels] in the state
+// pool (zeros when the sequence starts at position 0), which then takes the last taps - 1 inputs.  act: 0 none, 1 silu.  Sequences as in
+// StateMixParams (cu_q, k_len, seq_slot / slot0, active / park_slot, state, slot_stride, layer_offset)
+int    launch_short_conv(float* y, int ldy, const float* x, int ldx, int x_col, const float* w, int channels, int taps, int act,
+                         const StateMixParams& seqs, hipStream_t st);
 int    launch_gated_group_norm(void* y, int ldy, int out_elem_bytes, const float* x, int ldx, const float* w, const float* gate, int ldg, int rows,
                                int groups, int n, float eps, hipStream_t st);
+// y[row][h n + i] = o / sqrt(mean_i(o^2) + eps) * mult, o = a[row][h n + i] - lambda[0] * a[row][(heads + h) n + i]: the two maps of
+// differential attention (map-major heads, fp32) joined per head
+int launch_diff_head_norm(void* y, int ldy, int out_elem_bytes, const float* a, int lda, const float* lambda, float mult, int rows, int heads, int n,
+                          float eps, hipStream_t st);
+// y[row][i] = x[row][i] * sigmoid(gate[row][i]), i < n (x, gate fp32)
+int launch_sigmoid_gate_mul(void* y, int ldy, int out_elem_bytes, const float* x, int ldx, const float* gate, int ldg, int rows, int n, hipStream_t st);
+// x[i] = cap * tanh(x[i] / cap)
+int launch_softcap_f32(float* x, size_t n, float cap, hipStream_t st);
 // fp32 [n][V] -> fp16 [n][ld] (the sampler's logits rows)
 int launch_f32_to_f16_rows(half_t* out, int ld, const float* in, int n, int V, hipStream_t st);
 

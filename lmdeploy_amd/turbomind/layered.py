@@ -25,7 +25,7 @@ import numpy as np
 from .. import _ffi
 from .engine import Engine
 
-MIXER_ATTENTION, MIXER_LATENT, MIXER_LIGHTNING, MIXER_DELTA = 1, 2, 3, 4
+MIXER_ATTENTION, MIXER_LATENT, MIXER_LIGHTNING, MIXER_DELTA, MIXER_PARALLEL = 1, 2, 3, 4, 5
 MLP_NONE, MLP_DENSE, MLP_GATED, MLP_MOE = 0, 1, 2, 3
 ACT_RELU2, ACT_GELU_TANH, ACT_SILU, ACT_XIELU = 0, 1, 2, 3
 DTYPES = {'bfloat16': 0, 'bf16': 0, 'float32': 1, 'f32': 1}
@@ -73,6 +73,24 @@ class LayerSpec:
     router_softmax: bool = False  # soft-max scores weight the experts' outputs (times router_scale)
     router_scale: float = 1.0
     shared_ff: int = 0            # > 0: an expert of this size runs for every token
+    norm_groups: int = 0          # > 0 (post_norm blocks): the norm behind a sublayer is an RMS norm in that many groups, no bias
+    conv_taps: int = 0            # > 0: q, k, v pass a short causal convolution over time
+    diff_maps: bool = False       # differential attention: two score maps per head over the same values
+    diff_init: float = 0.0
+    rot_pairs: bool = False       # the rotation pairs channel 2i with 2i + 1
+    yarn_factor: float = 0.0      # > 0: slow rotation frequencies are divided by it (ramp between yarn_fast and yarn_slow turns over
+    yarn_original: float = 0.0    # yarn_original positions), cos and sin times 0.1 ln(factor) + 1
+    yarn_fast: float = 0.0
+    yarn_slow: float = 0.0
+    dist_buckets: int = 0         # parallel, left mixer: rows of the distance-bias table
+    dist_max: float = 0.0         # ... and the distance at which its logarithmic buckets end
+    r_heads: int = 0              # parallel, right mixer (gated delta rule): sizes
+    r_kv_heads: int = 0
+    r_dim: int = 0
+    r_vdim: int = 0
+    r_conv: int = 0
+    a_rank: int = 0               # inner sizes of the decay's and the gate's two-matrix projections
+    g_rank: int = 0
 
 
 @dataclass
@@ -89,6 +107,9 @@ class LayeredConfig:
     max_position_embeddings: int = 8192
     loop_times: int = 0           # > 0: tensors loop.in / loop.step exist
     final_layer_norm: bool = False  # the last norm is a layer norm with bias
+    embed_scale: float = 1.0      # multiplies the embedding output
+    logit_softcap: float = 0.0    # > 0: logits <- cap * tanh(logits / cap)
+    norm_groups: int = 0          # > 0: the last norm is an RMS norm in that many groups
     names: list = field(default_factory=list)   # tensor prefix of every layer run with tensors of its own ('' -> 'l<index>.')
 
     def native(self, dtype: str):
@@ -106,10 +127,13 @@ class LayeredConfig:
                            int(s.sink), s.mlp, s.ff, s.act, int(s.one_norm), int(s.resid_gate), s.loop_pass, int(s.qk_unit_norm),
                            int(s.v_unit_norm), int(s.dist_bias), int(s.out_gate), s.chunk, s.kv_rank, s.rot_dim, s.rot_base, s.experts, s.top, s.rot_dims,
                            int(s.post_norm), int(s.qkv_bias), int(s.qk_norm_w), s.rot_scale, s.window, s.keep_first, decays(s), s.decay_rank,
-                           int(s.expert_plain), int(s.router_softmax), s.router_scale, s.shared_ff)
+                           int(s.expert_plain), int(s.router_softmax), s.router_scale, s.shared_ff,
+                           s.norm_groups, s.conv_taps, int(s.diff_maps), s.diff_init, int(s.rot_pairs), s.yarn_factor, s.yarn_original, s.yarn_fast,
+                           s.yarn_slow, s.dist_buckets, s.dist_max, s.r_heads, s.r_kv_heads, s.r_dim, s.r_vdim, s.r_conv, s.a_rank, s.g_rank)
             for s in self.layers])
         return _ffi.LayeredConfig(self.width, self.vocab, len(self.layers), arr, self.norm_eps, self.norm_offset, self.residual_mult,
-                                  self.logit_scale, DTYPES[dtype], self.loop_times, int(self.final_layer_norm)), (arr, keep)
+                                  self.logit_scale, DTYPES[dtype], self.loop_times, int(self.final_layer_norm), self.embed_scale,
+                                  self.logit_softcap, self.norm_groups), (arr, keep)
 
     def tensor_name(self, run: int, leaf: str) -> str:
         """checkpoint name of tensor `leaf` of layer run `run` (the engine's slots count layer RUNS; a looped model's file counts layers)"""
@@ -118,7 +142,7 @@ class LayeredConfig:
     def tensor_shapes(self) -> dict:
         """{tensor name: shape} a checkpoint of this config holds"""
         W, out = self.width, {'embed': (self.vocab, self.width), 'final.norm': (self.width,), 'head': (self.vocab, self.width)}
-        if self.final_layer_norm:
+        if self.final_layer_norm and not self.norm_groups:
             out['final.norm.b'] = (W,)
         if self.loop_times > 0:
             out['loop.in'], out['loop.step'] = (W, 2 * W), (self.loop_times, W)
@@ -127,6 +151,9 @@ class LayeredConfig:
                 continue
             p = f'l{i}.'
             out[p + 'norm1'] = (W,)
+            if s.post_norm and s.norm_groups:
+                out.update(_group_shapes(p, s, W))
+                continue
             if s.post_norm:
                 out.update(_post_shapes(p, s, W))
                 continue
@@ -203,6 +230,101 @@ def _post_shapes(p: str, s: LayerSpec, W: int) -> dict:
         if s.shared_ff:
             out[p + 'mlp.shared.up'], out[p + 'mlp.shared.down'] = (s.shared_ff, W), (W, s.shared_ff)
     return out
+
+
+def _group_shapes(p: str, s: LayerSpec, W: int) -> dict:
+    """tensors of a post-norm block with RMS group norms: differential attention with convolved projections, or the parallel pair of a
+    biased attention and a gated delta rule; gated feed-forward"""
+    H, G, d, dv = s.heads, s.kv_heads, s.dim, s.vdim
+    out = {}
+    if s.mixer == MIXER_ATTENTION:
+        maps = 2 if s.diff_maps else 1
+        for t, n in (('q', H * maps * d), ('k', G * maps * d), ('v', G * dv)):
+            out[p + 'mix.' + t] = (n, W)
+            if s.conv_taps:
+                out[p + f'mix.{t}.conv'] = (n, s.conv_taps)
+        if s.qk_norm_w:
+            out[p + 'mix.q.norm'], out[p + 'mix.k.norm'] = (d,), (d,)
+        if s.diff_maps:
+            for t in ('lq1', 'lk1', 'lq2', 'lk2'):
+                out[p + 'mix.' + t] = (d,)
+        out[p + 'mix.o'] = (W, H * dv)
+    elif s.mixer == MIXER_PARALLEL:
+        a, b = p + 'mix.left.', p + 'mix.right.'
+        out.update({a + 'q': (H * d, W), a + 'k': (G * d, W), a + 'q.norm': (H * d,), a + 'k.norm': (G * d,), a + 'rel': (s.dist_buckets, H),
+                    a + 'talk': (H, H), a + 'g': (H * dv, W), a + 'o': (W, H * dv), a + 'out': (W,), b + 'out': (W,)})
+        Hr, Gr, dr, dvr = s.r_heads, s.r_kv_heads, s.r_dim, s.r_vdim
+        for t, n in (('q', Gr * dr), ('k', Gr * dr), ('v', Hr * dvr)):
+            out[b + t], out[b + t + '.conv'] = (n, W), (n, s.r_conv)
+        out.update({b + 'b': (Hr, W), b + 'A_log': (Hr,), b + 'norm': (dvr,), b + 'a1': (s.a_rank, W), b + 'a2': (Hr * dr, s.a_rank),
+                    b + 'dt_bias': (Hr * dr,), b + 'g1': (s.g_rank, W), b + 'g2': (Hr * dvr, s.g_rank), b + 'o': (W, Hr * dvr)})
+    else:
+        raise NotImplementedError(f'{p}: mixer {s.mixer} in a block with group norms')
+    if s.mlp:
+        out[p + 'norm2'] = (W,)
+        out[p + 'mlp.gate'], out[p + 'mlp.up'], out[p + 'mlp.down'] = (s.ff, W), (s.ff, W), (W, s.ff)
+    return out
+
+
+def _mededra_layer(i: int, L: dict, shapes: dict, groups: int) -> LayerSpec:
+    m, mlp, kind = L['mixer'], L.get('mlp'), L['type']
+    s = LayerSpec(post_norm=True, norm_groups=groups)
+    if kind == 'attention':
+        s.mixer, s.heads, s.dim = MIXER_ATTENTION, int(m['heads']), int(m['dim'])
+        s.kv_heads, s.vdim = int(m.get('kv_heads', s.heads)), int(m.get('vdim', s.dim))
+        s.scale = float(m['scale']) if 'scale' in m else s.dim ** -0.5
+        s.softcap = float(m.get('softcap') or 0.0)
+        s.qk_norm_w, s.diff_maps, s.diff_init = True, True, float(m['diff'])
+        s.conv_taps = int(m.get('conv') or 0)
+        s.window = int((m.get('mask') or {}).get('size') or 0)
+        rot = m.get('rot') or {}
+        if rot:
+            s.rot_pairs, s.rot_dims, s.rot_base = True, int(rot.get('dims', s.dim)), float(rot['base'])
+            sc = rot.get('scaling') or {}
+            if sc:
+                s.yarn_factor, s.yarn_original = float(sc['factor']), float(sc['original'])
+                s.yarn_fast, s.yarn_slow = float(sc['fast']), float(sc['slow'])
+            if s.rot_dims % 2 or not 0 <= s.rot_dims <= s.dim:
+                raise ValueError(f'layer {i}: rot.dims must be even and at most dim')
+    elif kind == 'parallel':
+        a, b = m['left'], m['right']
+        s.mixer, s.heads, s.dim = MIXER_PARALLEL, int(a['heads']), int(a['dim'])
+        s.kv_heads, s.vdim = int(a.get('kv_heads', s.heads)), int(a.get('vdim', s.dim))
+        s.scale = float(a['scale']) if 'scale' in a else s.dim ** -0.5
+        s.window = int((a.get('mask') or {}).get('size') or 0)
+        s.dist_max = float(a['bias_max'])
+        rel = shapes.get(f'l{i}.mix.left.rel')          # the number of buckets, and the inner sizes below, are the tensors' own
+        s.dist_buckets = int(rel[0]) if rel else int(a.get('buckets', 0))
+        if s.vdim != s.dim:
+            raise ValueError(f'layer {i}: the left mixer\'s values are its keys: vdim = dim')
+        s.r_heads, s.r_dim = int(b['heads']), int(b['dim'])
+        s.r_kv_heads, s.r_vdim, s.r_conv = int(b.get('kv_heads', s.r_heads)), int(b.get('vdim', s.r_dim)), int(b.get('conv') or 1)
+        a1, g1 = shapes.get(f'l{i}.mix.right.a1'), shapes.get(f'l{i}.mix.right.g1')
+        s.a_rank = int(a1[0]) if a1 else int(b.get('a_rank', 0))
+        s.g_rank = int(g1[0]) if g1 else int(b.get('g_rank', 0))
+    else:
+        raise NotImplementedError(f'layer {i}: mixer {kind!r}')
+    if mlp is None:
+        return s
+    if mlp.get('kind') != 'dense':
+        raise NotImplementedError(f'layer {i}: feed-forward kind {mlp.get("kind")!r}')
+    s.mlp, s.ff, s.act = MLP_GATED, int(mlp['ff']), ACT_SILU
+    return s
+
+
+def _mededra(c: dict, shapes: dict | None = None) -> LayeredConfig:
+    """Mededra: blocks x += GN1(mixer(x)); x += GN2(ff(x)) with RMS norms in groups on the sublayers' results.  Mixers: differential
+    attention (two score maps per head, q / k / v through a short causal convolution, a weighted norm per map, pairwise rotation with
+    scaled frequencies, capped scores, a sliding window), or a parallel pair -- windowed attention whose values are its keys, with a
+    bucketed distance bias, scores mixed between heads, one added to the soft-max denominator and a gated output, beside a gated delta
+    rule -- whose normed results are averaged.  Gated silu feed-forward, scaled embedding, capped logits.  `shapes` ({tensor name: shape}
+    of the checkpoint) settles the sizes the config leaves to the tensors (distance buckets, inner sizes of two-matrix projections)."""
+    groups = int(c['norm'].get('groups', 1))
+    layers = [_mededra_layer(i, L, shapes or {}, groups) for i, L in enumerate(c['layers'])]
+    return LayeredConfig(arch='Mededra', width=int(c['width']), vocab=int(c['vocab']), layers=layers, norm_eps=float(c['norm']['eps']),
+                         norm_offset=0.0, residual_mult=1.0, logit_scale=1.0, eos_token_id=c.get('eos_token_id'),
+                         embed_scale=float((c.get('embedding') or {}).get('scale', 1.0)), logit_softcap=float(c.get('logit_softcap') or 0.0),
+                         norm_groups=groups)
 
 
 def _febivik_layer(i: int, L: dict, shapes: dict) -> LayerSpec:
@@ -342,8 +464,8 @@ def _fokonex(c: dict) -> LayeredConfig:
                          logit_scale=float(c['logit_scale']), eos_token_id=c.get('eos_token_id'))
 
 
-FAMILIES = {'Fokonex': _fokonex, 'Bedenex': _bedenex, 'Febivik': _febivik}
-NEEDS_SHAPES = {'Febivik'}     # readers that take the checkpoint's tensor shapes as a second argument
+FAMILIES = {'Fokonex': _fokonex, 'Bedenex': _bedenex, 'Febivik': _febivik, 'Mededra': _mededra}
+NEEDS_SHAPES = {'Febivik', 'Mededra'}     # readers that take the checkpoint's tensor shapes as a second argument
 
 
 def is_layered(model_path: str) -> bool:
