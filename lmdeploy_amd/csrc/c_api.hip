@@ -710,6 +710,7 @@ int tm_general_attention(const tm_general_attn* a, tm_stream_t st)
     p.dist_r1 = a->dist_r1, p.dist_r2 = a->dist_r2, p.chunk = a->chunk, p.out_gate = a->out_gate, p.ld_gate = a->ld_gate;
     p.out_head_stride = a->out_head_stride;
     p.window = a->window, p.keep_first = a->keep_first;
+    p.k_heads = a->k_heads, p.v_heads = a->v_heads, p.dist_table = a->dist_table, p.dist_table_len = a->dist_table_len, p.out_f32 = a->out_f32;
     if (a->store_kv) {
         TM_REQUIRE(a->kv, "store_kv without kv rows");
         const int rc = launch_kv_store_general(a->kv, a->ldkv, a->k_col, a->v_col, p, (hipStream_t)st);

@@ -355,7 +355,8 @@ int launch_rows_prepare(int* row_seq, int* row_pos, const int* cu_q, const int* 
 template<class T>
 __global__ void kv_store_general_kernel(const T* __restrict__ qkv, int ld, int k_col, int v_col, GeneralAttnParams p)
 {
-    const int per = p.kv_heads * (p.dim + p.vdim);
+    const int kh = p.k_heads > 0 ? p.k_heads : p.kv_heads, vh = p.v_heads > 0 ? p.v_heads : p.kv_heads;
+    const int per = kh * p.dim + vh * p.vdim;
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= (size_t)p.rows * per) {
         return;
@@ -364,7 +365,7 @@ __global__ void kv_store_general_kernel(const T* __restrict__ qkv, int ld, int k
     const int s = p.row_seq[t], pos = p.row_pos[t];
     char* base = (char*)p.block_ptrs[(size_t)(p.seq_slot ? p.seq_slot[s] : s) * p.block_stride + pos / p.block_len] + p.layer_offset;
     const int ti = pos % p.block_len;
-    const int nk = p.kv_heads * p.dim;
+    const int nk = kh * p.dim;
     if (c < nk) {
         const int g = c / p.dim, d = c % p.dim;
         ((T*)base)[((size_t)g * p.block_len + ti) * p.dim + d] = qkv[(size_t)t * ld + k_col + c];
@@ -378,7 +379,8 @@ __global__ void kv_store_general_kernel(const T* __restrict__ qkv, int ld, int k
 int launch_kv_store_general(const void* qkv, int ld, int k_col, int v_col, const GeneralAttnParams& p, hipStream_t st)
 {
     TM_REQUIRE(qkv && p.row_seq && p.row_pos && p.block_ptrs && p.block_stride >= 1, "kv_store_general: operands");
-    const size_t n = (size_t)p.rows * p.kv_heads * (p.dim + p.vdim);
+    const int    kh = p.k_heads > 0 ? p.k_heads : p.kv_heads, vh = p.v_heads > 0 ? p.v_heads : p.kv_heads;
+    const size_t n = (size_t)p.rows * (kh * p.dim + vh * p.vdim);
     if (n == 0) {
         return 0;
     }

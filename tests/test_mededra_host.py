@@ -1,0 +1,144 @@
+"""Host tests of the Mededra design: the config reader's mapping of every constant, the sizes it takes from the checkpoint's tensors,
+and hand cases of the float64 oracle's mechanisms (tests/mededra_oracle.py)."""
+import math
+
+import numpy as np
+import pytest
+
+from lmdeploy_amd.turbomind import layered
+from tests import mededra_oracle as mo
+
+SCALING = {'factor': 4.0, 'original': 64, 'fast': 8.0, 'slow': 1.0}
+
+
+def _cfg():
+    return mo.make_config(48, 101, [
+        mo.attention_layer(4, 2, 8, 12, 0.3, 50, 6, 3000.0, SCALING, 9.0, 0.35, 4, mo.dense(40)),
+        mo.parallel_layer(mo.left_mixer(6, 2, 8, 40, 100, 0.25), mo.right_mixer(4, 2, 10, 12, 2)),
+    ], eps=1e-6, groups=3, embed_scale=2.5, logit_softcap=11.0)
+
+
+def test_reader_maps_every_constant(tmp_path):
+    cfg = _cfg()
+    w = mo.random_weights(cfg, 0, buckets=10, a_rank=5, g_rank=7)
+    mo.write_checkpoint(str(tmp_path), cfg, w)
+    c = layered.read_layered_config(str(tmp_path))
+    assert (c.arch, c.width, c.vocab, c.norm_groups, c.embed_scale, c.logit_softcap) == ('Mededra', 48, 101, 3, 2.5, 11.0)
+    assert abs(c.norm_eps - 1e-6) < 1e-12 and not c.final_layer_norm
+    a, b = c.layers
+    assert (a.mixer, a.heads, a.kv_heads, a.dim, a.vdim, a.window, a.conv_taps) == (layered.MIXER_ATTENTION, 4, 2, 8, 12, 50, 4)
+    assert a.post_norm and a.norm_groups == 3 and a.diff_maps and a.diff_init == 0.35 and a.qk_norm_w and a.rot_pairs
+    assert (a.rot_dims, a.rot_base, a.softcap, a.scale) == (6, 3000.0, 9.0, 0.3)
+    assert (a.yarn_factor, a.yarn_original, a.yarn_fast, a.yarn_slow) == (4.0, 64.0, 8.0, 1.0)
+    assert (a.mlp, a.ff, a.act) == (layered.MLP_GATED, 40, layered.ACT_SILU)
+    assert (b.mixer, b.heads, b.kv_heads, b.dim, b.vdim, b.window, b.scale, b.dist_max) == (layered.MIXER_PARALLEL, 6, 2, 8, 8, 40, 0.25, 100.0)
+    assert (b.r_heads, b.r_kv_heads, b.r_dim, b.r_vdim, b.r_conv) == (4, 2, 10, 12, 2)
+    assert (b.dist_buckets, b.a_rank, b.g_rank) == (10, 5, 7)       # the tensors' own sizes
+    assert b.mlp == layered.MLP_NONE and b.conv_taps == 0 and not b.diff_maps
+    shapes = c.tensor_shapes()
+    assert shapes == {k: tuple(np.shape(v)) for k, v in w.items()}
+    native, keep = c.native('float32')
+    assert native.n_layers == 2 and native.layers[1].r_vdim == 12 and native.norm_groups == 3
+
+
+def test_group_norm_scales_each_part_by_its_own_rms():
+    x = np.array([[3.0, 4.0, 0.0, 0.5]])
+    y = mo.group_norm(x, np.array([1.0, 1.0, 2.0, 2.0]), 2, 0.0)
+    r0, r1 = math.sqrt(12.5), math.sqrt(0.125)
+    assert np.allclose(y, [[3 / r0, 4 / r0, 0.0, 1.0 / r1]])
+    assert np.allclose(mo.group_norm(x, np.ones(4), 1, 0.0), x / math.sqrt((9 + 16 + 0.25) / 4))
+
+
+def test_short_conv_reads_back_in_time_and_continues_from_its_last_inputs():
+    u = np.arange(1.0, 7.0)[:, None] * np.array([[1.0, 10.0]])
+    wc = np.array([[0.5, 0.25, 2.0], [1.0, 0.0, -1.0]])             # the last column meets the current token
+    y = mo.short_conv(u, wc)
+    assert np.allclose(y[0], [2.0 * 1, -10.0]) and np.allclose(y[1], [0.25 * 1 + 2.0 * 2, -20.0])
+    assert np.allclose(y[3], [0.5 * 2 + 0.25 * 3 + 2.0 * 4, 20.0 - 40.0])
+    for cut in (1, 2, 4):                                            # a portion continues from the two inputs ahead of it
+        before = np.concatenate([np.zeros((2, 2)), u[:cut]])[-2:]
+        assert np.allclose(mo.short_conv(u[cut:], wc, before), y[cut:])
+
+
+def test_rotation_pairs_neighbours_and_scales_slow_frequencies():
+    f, mult = mo.yarn_frequencies(8, 100.0, None)
+    assert np.allclose(f, 100.0 ** (-np.arange(4) / 4.0)) and mult == 1.0
+    f2, mult2 = mo.yarn_frequencies(8, 100.0, {'factor': 4.0, 'original': 64, 'fast': 8.0, 'slow': 1.0})
+    # channel pair turning 8 times over 64 positions: c = 8 ln(64 / (16 pi)) / (2 ln 100) = 0.21 -> lo 0; once: c = 2.02 -> hi 3
+    ramp = np.clip(np.arange(4) / 3.0, 0, 1)
+    assert np.allclose(f2, f / 4.0 * ramp + f * (1 - ramp)) and abs(mult2 - (0.1 * math.log(4.0) + 1.0)) < 1e-12
+    x = np.zeros((1, 1, 6))
+    x[0, 0] = [1.0, 0.0, 0.0, 2.0, 5.0, 7.0]
+    y = mo.rotate_pairs(x, [3], 4, 100.0, None)
+    a0, a1 = 3.0, 3.0 * 100.0 ** -0.5
+    assert np.allclose(y[0, 0], [math.cos(a0), math.sin(a0), -2 * math.sin(a1), 2 * math.cos(a1), 5.0, 7.0])
+
+
+def test_distance_buckets():
+    B, D = 16, 240.0
+    assert [mo.distance_bucket(n, B, D) for n in range(8)] == list(range(8))
+    assert mo.distance_bucket(8, B, D) == 8 and mo.distance_bucket(12, B, D) == 8      # 8 ln(1.5) / ln(30) = 0.95
+    assert mo.distance_bucket(13, B, D) == 9 and mo.distance_bucket(239, B, D) == 15 and mo.distance_bucket(100000, B, D) == 15
+    assert [mo.distance_bucket(n, 4, 8.0) for n in (0, 1, 2, 3, 4, 7, 8)] == [0, 1, 2, 2, 3, 3, 3]
+
+
+def test_softmax_with_one_in_the_denominator_and_window():
+    s = np.array([[0.0, 0.0, 0.0], [math.log(3.0), 0.0, 5.0]])
+    mask = mo.window_mask(3, 2)[1:]
+    assert mask.tolist() == [[True, True, False], [False, True, True]]
+    p = mo.softmax_rows(s, np.array([[True, True, False], [True, True, False]]), plus_one=True)
+    assert np.allclose(p, [[1 / 3, 1 / 3, 0], [3 / 5, 1 / 5, 0]])
+    assert np.allclose(mo.softmax_rows(s[:1], np.array([[True, True, False]])), [[0.5, 0.5, 0]])
+
+
+def test_gated_delta_recurrence_hand_cases():
+    k = np.array([[1.0, 0.0], [0.0, 1.0], [1.0, 0.0]])
+    v = np.array([[2.0, 3.0], [5.0, 7.0], [11.0, 13.0]])
+    one = np.ones((3, 2))
+    o, S = mo.gated_delta_recurrence(k, k, v, one, np.ones(3))       # full write strength, no decay: a key's row is replaced by its value
+    assert np.allclose(o, v) and np.allclose(S, [[11.0, 13.0], [5.0, 7.0]])
+    o, S = mo.gated_delta_recurrence(k, k, v, one, np.full(3, 0.5))  # half strength: the row moves half way to the value
+    assert np.allclose(S[0], 0.5 * (0.5 * v[0]) + 0.5 * v[2]) and np.allclose(o[2], S[0])
+    g = np.array([[1.0, 1.0], [0.5, 1.0], [0.5, 0.25]])             # the decay scales the key channels' rows BEFORE the token's write
+    o, S = mo.gated_delta_recurrence(k, k, v, g, np.array([1.0, 0.0, 0.0]))
+    assert np.allclose(S, [[2.0 * 0.25, 3.0 * 0.25], [0.0, 0.0]]) and np.allclose(o[1], [0.0, 0.0]) and np.allclose(o[2], S[0])
+    a, Sa = mo.gated_delta_recurrence(k[:2], k[:2], v[:2], g[:2], np.array([0.3, 0.9]))
+    b, Sb = mo.gated_delta_recurrence(k[2:], k[2:], v[2:], g[2:], np.array([0.6]), Sa)
+    c, Sc = mo.gated_delta_recurrence(k, k, v, g, np.array([0.3, 0.9, 0.6]))
+    assert np.allclose(np.concatenate([a, b]), c) and np.allclose(Sb, Sc)
+
+
+def test_differential_attention_subtracts_the_second_map():
+    cfg = mo.make_config(16, 11, [mo.attention_layer(1, 1, 4, 4, 0.5, 0, 0, conv=1)])
+    w = mo.random_weights(cfg, 5)
+    p = 'l0.mix.'
+    for t in ('q.conv', 'k.conv', 'v.conv'):
+        w[p + t] = np.ones_like(w[p + t])
+    for t in ('lq1', 'lk1', 'lq2', 'lk2'):
+        w[p + t] = np.zeros(4)
+    assert mo.diff_lambda(w, p, 0.5) == 0.5                          # e^0 - e^0 + diff
+    w[p + 'lq1'], w[p + 'lk1'] = np.array([1.0, 0, 0, 0]), np.array([math.log(2.0), 0, 0, 0])
+    assert abs(mo.diff_lambda(w, p, 0.25) - (2.0 - 1.0 + 0.25)) < 1e-12
+    h = np.random.default_rng(0).normal(0, 1, (5, 16))
+    w[p + 'q'][4:] = w[p + 'q'][:4]                                  # both maps alike: o = (1 - lambda) a, whose unit RMS form times (1 - diff)
+    w[p + 'k'][4:] = w[p + 'k'][:4]
+    w[p + 'o'] = np.eye(16)[:, :4]
+    y = mo.diff_attention_mixer(h, cfg['layers'][0]['mixer'], w, p, 1e-9)
+    assert np.allclose(np.sqrt((y[:, :4] ** 2).mean(-1)), 0.5, atol=1e-6)
+    assert np.allclose(y[0, :4] / np.abs(y[0, :4]).max(), (h[0] @ w[p + 'v'].T) / np.abs(h[0] @ w[p + 'v'].T).max() * np.sign(1 - mo.diff_lambda(w, p, 0.5)))
+
+
+def test_a_block_adds_the_normed_sublayer_result():
+    cfg = _cfg()
+    w = mo.random_weights(cfg, 2, buckets=10, a_rank=5, g_rank=7)
+    toks = [3, 7, 1, 100, 42, 7]
+    logits, trail = mo.forward(cfg, w, toks, True)
+    assert logits.shape == (6, 101) and trail.shape == (2, 6, 48) and np.abs(logits).max() < 11.0
+    x0 = w['embed'][toks] * 2.5
+    y = mo.diff_attention_mixer(x0, cfg['layers'][0]['mixer'], w, 'l0.mix.', 1e-6)
+    x1 = x0 + mo.group_norm(y, w['l0.norm1'], 3, 1e-6)
+    x1 = x1 + mo.group_norm(mo.gated_ff(x1, w, 'l0.mlp.'), w['l0.norm2'], 3, 1e-6)
+    assert np.allclose(trail[0], x1)
+    assert np.allclose(mo.forward(cfg, w, toks[:4]), logits[:4])     # causal
+    with pytest.raises(NotImplementedError):
+        layered.FAMILIES['Mededra']({'width': 8, 'vocab': 8, 'norm': {'eps': 1e-5}, 'layers': [{'type': 'other', 'mixer': {}}]})
