@@ -343,9 +343,9 @@ def main():
                          'shapes of real decoders beside the fp16 Llama-family engine at equal size (lmdeploy_amd/turbomind/layered_bench.py); '
                          'prints its own JSON line; 1 GPU')
     ap.add_argument('--layered-sizes', default='', help='with --layered: comma-separated subset of w2048,w4096')
-    ap.add_argument('--layered-design', default='fokonex', choices=['fokonex', 'bedenex', 'febivik'],
-                    help='with --layered: fokonex (beside the fp16 Llama-family engine), bedenex (beside the Fokonex blocks at equal size) or '
-                         'febivik (beside the Bedenex blocks at equal size)')
+    ap.add_argument('--layered-design', default='fokonex', choices=['fokonex', 'bedenex', 'febivik', 'mededra'],
+                    help='with --layered: fokonex (beside the fp16 Llama-family engine), bedenex (beside the Fokonex blocks at equal size), '
+                         'febivik (beside the Bedenex blocks at equal size) or mededra (beside the Febivik blocks at equal size)')
     ap.add_argument('--cpu-config0', action='store_true',
                     help='BASELINE.json configs[0] only: InternLM2-1.8B fp16 greedy decode on the host cores (oracle/cpu_baseline.py::run_config0, the '
                          'torch-CPU port of the reference\'s default-backend ops); prints its own JSON line; no GPU is touched')
@@ -358,7 +358,7 @@ def main():
         r = layered_bench.run(steps, args.warmup, batch, args.prompt_len, [x for x in args.layered_sizes.split(',') if x] or None,
                               args.layered_design, args.layered_one)
         first, beside = {'fokonex': ('fokonex_bf16', 'the fp16 Llama-family engine'), 'bedenex': ('bedenex_bf16', 'Fokonex blocks'),
-                         'febivik': ('febivik_bf16', 'Bedenex blocks')}[args.layered_design]
+                         'febivik': ('febivik_bf16', 'Bedenex blocks'), 'mededra': ('mededra_bf16', 'Febivik blocks')}[args.layered_design]
         emit_json({'metric': f'prefill and decode tokens/sec of a {args.layered_design.capitalize()} layer-list model (bf16) beside {beside} at equal size, '
                              f'decode batch {batch}, context {args.prompt_len}', 'value': round(next(iter(r.values()))[first]['decode_tokens_per_s'], 1),
                    'unit': 'tokens/s', 'n_gpus': 1, 'steps': steps, 'warmup': args.warmup, 'higher_is_better': True, 'dtype': 'bf16', 'data': 'synthetic',

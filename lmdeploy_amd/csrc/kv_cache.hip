@@ -481,15 +481,18 @@ int launch_attn_prep(const float* proj, int ld, int q_col, int k_col, int v_col,
     return 0;
 }
 
-// attention with mixed heads as attention over one wide key (see launch_talk_prep): one workgroup per row
+// attention with mixed heads as attention over one wide key (see launch_talk_prep): grid (rows, head blocks) -- a workgroup forms the mixed
+// queries of HB heads of one row (every workgroup computes the row's two norm statistics itself); head block 0 also writes the cache entry
 template<class T>
 __global__ __launch_bounds__(256) void talk_prep_kernel(const float* __restrict__ proj, int ld, int q_col, int k_col, T* __restrict__ q_out, int ldq,
                                                         const float* __restrict__ q_w, const float* __restrict__ k_w,
-                                                        const float* __restrict__ talk, int D, float eps, GeneralAttnParams p)
+                                                        const float* __restrict__ talk, int D, int HB, float eps, GeneralAttnParams p)
 {
-    extern __shared__ float tp_lds[];  // the normed queries [H][D]
+    extern __shared__ float tp_lds[];  // the normed queries [H][D], then the mixing rows of this block's heads [HB][H]
     __shared__ float red[4];
     const int    t = blockIdx.x, H = p.q_heads, G = p.kv_heads, r = H / G, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int    h0 = blockIdx.y * HB, nh = min(HB, H - h0);
+    float*       tk = tp_lds + H * D;
     const float *q = proj + (size_t)t * ld + q_col, *k = proj + (size_t)t * ld + k_col;
     auto block_sum = [&](float v) {
         v = group_sum<64>(v);
@@ -512,15 +515,21 @@ __global__ __launch_bounds__(256) void talk_prep_kernel(const float* __restrict_
     for (int i = threadIdx.x; i < H * D; i += 256) {
         tp_lds[i] = q[i] * qinv * q_w[i];
     }
+    for (int i = threadIdx.x; i < nh * H; i += 256) {
+        tk[i] = talk[(size_t)h0 * H + i];
+    }
     __syncthreads();
     // Q'[h][c D + d] = sum over the heads g of group c of talk[h][g] q_g[d]
-    for (int i = threadIdx.x; i < H * G * D; i += 256) {
-        const int h = i / (G * D), c = (i / D) % G, d = i % D;
+    for (int i = threadIdx.x; i < nh * G * D; i += 256) {
+        const int hl = i / (G * D), c = (i / D) % G, d = i % D;
         float     acc = 0.f;
         for (int g = c * r; g < (c + 1) * r; ++g) {
-            acc = fmaf(talk[h * H + g], tp_lds[g * D + d], acc);
+            acc = fmaf(tk[hl * H + g], tp_lds[g * D + d], acc);
         }
-        q_out[(size_t)t * ldq + i] = (T)acc;
+        q_out[(size_t)t * ldq + (size_t)h0 * G * D + i] = (T)acc;
+    }
+    if (blockIdx.y != 0) {
+        return;
     }
     const int s = p.row_seq[t], pos = p.row_pos[t], ti = pos % p.block_len;
     char*     base = (char*)p.block_ptrs[(size_t)(p.seq_slot ? p.seq_slot[s] : s) * p.block_stride + pos / p.block_len] + p.layer_offset;
@@ -543,12 +552,18 @@ int launch_talk_prep(const float* proj, int ld, int q_col, int k_col, void* q_ou
     if (p.rows == 0) {
         return 0;
     }
-    const size_t lds = (size_t)p.q_heads * head_dim * 4;
+    // few rows (decoded tokens): one head per workgroup so that the launch still fills the device; many rows: as few head blocks as keep
+    // the mixing rows in LDS, the norm statistics are then computed once per row
+    const int H = p.q_heads;
+    int       hb = p.rows >= 512 ? H : std::max(1, (int)((int64_t)H * p.rows / 512));
+    hb           = std::min(hb, std::max(1, (15 * 1024 - H * head_dim) / H));
+    const size_t lds = ((size_t)H * head_dim + (size_t)hb * H) * 4;
+    const dim3   grid(p.rows, (H + hb - 1) / hb);
     if (p.elem_bytes == 2) {
-        talk_prep_kernel<__bf16><<<p.rows, 256, lds, st>>>(proj, ld, q_col, k_col, (__bf16*)q_out, ldq, q_w, k_w, talk, head_dim, eps, p);
+        talk_prep_kernel<__bf16><<<grid, 256, lds, st>>>(proj, ld, q_col, k_col, (__bf16*)q_out, ldq, q_w, k_w, talk, head_dim, hb, eps, p);
     }
     else {
-        talk_prep_kernel<float><<<p.rows, 256, lds, st>>>(proj, ld, q_col, k_col, (float*)q_out, ldq, q_w, k_w, talk, head_dim, eps, p);
+        talk_prep_kernel<float><<<grid, 256, lds, st>>>(proj, ld, q_col, k_col, (float*)q_out, ldq, q_w, k_w, talk, head_dim, hb, eps, p);
     }
     TM_HIP_CHECK(hipGetLastError());
     return 0;

@@ -14,6 +14,11 @@ model the engine serves, the Fokonex blocks above, at equal width, heads, layer 
 tokens, xIELU and soft-max-routed squared-ReLU experts with a shared expert, layer norms behind the sublayers) beside the closest model
 the engine serves -- the Bedenex blocks above (routed experts, fused fp32 projections) -- at equal width, heads, layer count, vocabulary
 and active feed-forward parameters.
+
+`bench.py --layered --layered-design mededra`: Mededra blocks (differential attention with convolved projections, the parallel pair of a
+biased attention with mixed heads and a gated delta rule, RMS group norms behind the sublayers, gated silu feed-forward) beside the
+closest model the engine serves -- the Febivik blocks above (post-norm blocks, windowed attention, a delta-rule state mixer) -- at equal
+width, heads, layer count and vocabulary.
 """
 from __future__ import annotations
 
@@ -153,6 +158,57 @@ def _llama_engine(s, batch, session_len, max_prefill):
     return eng
 
 
+MEDEDRA = dict(window=2048, map_dim=64, rot_dims=64, conv=4, left_kv=2, buckets=32, bias_max=4096, rank=64)
+
+
+def mededra_config(s) -> dict:
+    """config.json of the benchmark model: [differential attention x 3, parallel pair] repeated, every block with the gated feed-forward of
+    the size's own `inter`.  Differential attention: two maps of 64 channels per head (the projections are as wide as heads of 128), values
+    of 128, window 2048, scaled pairwise rotation, 4-tap convolutions.  Parallel pair: left = windowed attention over 2 key heads of 128
+    (a wide key of 256) with the bucketed distance bias and mixed heads; right = gated delta rule with heads of 128 x 128"""
+    b, H, G = MEDEDRA, s['heads'], s['kv_heads']
+    att = {'heads': H, 'kv_heads': G, 'dim': b['map_dim'], 'vdim': 128, 'scale': b['map_dim'] ** -0.5, 'softcap': 30.0, 'diff': 0.5, 'conv': b['conv'],
+           'mask': {'size': b['window']},
+           'rot': {'base': 250000.0, 'dims': b['rot_dims'], 'scaling': {'factor': 8.0, 'original': 2048, 'fast': 32.0, 'slow': 1.0}}}
+    left = {'heads': H, 'kv_heads': b['left_kv'], 'dim': 128, 'vdim': 128, 'scale': 128 ** -0.5, 'mask': {'size': b['window']},
+            'bias_max': b['bias_max'], 'buckets': b['buckets']}
+    right = {'heads': H, 'kv_heads': G, 'dim': 128, 'vdim': 128, 'conv': b['conv'], 'a_rank': b['rank'], 'g_rank': b['rank']}
+    dense = {'kind': 'dense', 'ff': s['inter']}
+    four = [{'type': 'attention', 'mixer': att, 'mlp': dense}] * 3 + [{'type': 'parallel', 'mixer': {'left': left, 'right': right}, 'mlp': dense}]
+    return {'architecture': 'Mededra', 'width': s['width'], 'vocab': s['vocab'], 'norm': {'eps': 1e-5, 'groups': 8}, 'embedding': {'scale': 1.0},
+            'logit_softcap': 30.0, 'layers': [four[i % 4] for i in range(s['layers'])]}
+
+
+def _mededra_engine(s, batch, session_len, max_prefill):
+    from . import layered
+    cfg = layered.FAMILIES['Mededra'](mededra_config(s))
+    eng = layered.LayeredEngine(cfg, dtype='bfloat16', max_batch_size=batch, session_len=session_len, max_prefill_token_num=max_prefill)
+    eng.init_synthetic(seed=1)
+    eng.start()
+    return eng
+
+
+def _mededra_decode_bytes(s, batch, ctx):
+    """bytes each category of ONE decode step must move: every weight once, the cache entries inside the windows once per sequence, the
+    delta rule's state read and written once (fp32)"""
+    b, W, H, G, V = MEDEDRA, s['width'], s['heads'], s['kv_heads'], s['vocab']
+    out = dict(gemm_qkv=0, attention=0, gemm_o=0, gemm_gate_up=0, gemm_down=0, lm_head=2 * W * V)
+    seen = min(ctx, b['window'])
+    for i in range(s['layers']):
+        if i % 4 != 3:
+            out['gemm_qkv'] += 2 * W * (H * 2 * b['map_dim'] + G * 2 * b['map_dim'] + G * 128)
+            out['attention'] += 2 * batch * (G * 2 * b['map_dim'] + G * 128) * seen
+            out['gemm_o'] += 2 * W * H * 128
+        else:
+            lk = b['left_kv']
+            out['gemm_qkv'] += 2 * W * (H * 128 + lk * 128 + H * 128 + 2 * G * 128 + H * 128 + H + 2 * b['rank']) + 2 * b['rank'] * 2 * H * 128
+            out['attention'] += 2 * batch * 2 * lk * 128 * seen + batch * H * 128 * 128 * 4 * 2
+            out['gemm_o'] += 2 * 2 * W * H * 128
+        out['gemm_gate_up'] += 2 * W * 2 * s['inter']
+        out['gemm_down'] += 2 * W * s['inter']
+    return out
+
+
 def _measure(eng, vocab, batch, prompt_len, steps, warmup, prefill_seqs):
     rng = np.random.default_rng(0)
     out = {}
@@ -201,7 +257,8 @@ def run(steps: int, warmup: int, batch: int, prompt_len: int, sizes=None, design
     res = {}
     pair = {'fokonex': (('fokonex_bf16', _fokonex_engine), ('llama_f16', _llama_engine)),
             'bedenex': (('bedenex_bf16', _bedenex_engine), ('fokonex_bf16', _fokonex_engine)),
-            'febivik': (('febivik_bf16', _febivik_engine), ('bedenex_bf16', _bedenex_engine))}[design]
+            'febivik': (('febivik_bf16', _febivik_engine), ('bedenex_bf16', _bedenex_engine)),
+            'mededra': (('mededra_bf16', _mededra_engine), ('febivik_bf16', _febivik_engine))}[design]
     if only_first:
         pair = pair[:1]
     for name in (sizes or SIZES):
@@ -213,7 +270,7 @@ def run(steps: int, warmup: int, batch: int, prompt_len: int, sizes=None, design
             eng = make(s, batch, session_len, 8192)
             m = _measure(eng, s['vocab'], batch, prompt_len, steps, warmup, prefill_seqs)
             ctx = prompt_len + warmup + steps // 2
-            need = _febivik_decode_bytes(s, batch, ctx) if kind == 'febivik_bf16' else \
+            need = _mededra_decode_bytes(s, batch, ctx) if kind == 'mededra_bf16' else _febivik_decode_bytes(s, batch, ctx) if kind == 'febivik_bf16' else \
                 _bedenex_decode_bytes(s, batch, ctx) if kind == 'bedenex_bf16' else _decode_bytes(s, batch, ctx, kind == 'fokonex_bf16')
             m['decode_hbm_roofline_fraction'] = {k: round(need[k] / HBM_BYTES_PER_S / (m['decode_categories_ms'][k] * 1e-3), 4)
                                                  for k in need if m['decode_categories_ms'].get(k)}
