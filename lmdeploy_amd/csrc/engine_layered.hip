@@ -1411,7 +1411,7 @@ int tm_engine_create_layered(tm_engine** out, const tm_engine_config* c, const t
                        at + ": a block with group norms takes none of the other block forms' switches");
             TM_REQUIRE(s.heads >= 1 && s.kv_heads >= 1 && s.heads % s.kv_heads == 0 && s.dim >= 1 && s.dim <= 256 && s.vdim >= 1 && s.vdim <= 256 && s.window >= 0,
                        at + ": heads % kv_heads, 1 <= dim, vdim <= 256, window >= 0");
-            TM_REQUIRE(s.conv_taps >= 0 && s.conv_taps <= 8, at + ": at most 8 taps");
+            TM_REQUIRE(s.conv_taps >= 0 && s.conv_taps <= 16, at + ": at most 16 taps");
             TM_REQUIRE(s.mlp == TM_MLP_NONE || (s.mlp == TM_MLP_GATED && s.ff >= 1 && s.act >= TM_ACT_RELU2 && s.act <= TM_ACT_SILU), at + ": gated feed-forward");
             if (s.mixer == TM_MIXER_ATTENTION) {
                 TM_REQUIRE(s.rot_dims >= 0 && s.rot_dims % 2 == 0 && s.rot_dims <= s.dim && s.rot_base > 0.f && s.rot_scale > 0.f,
@@ -1424,8 +1424,8 @@ int tm_engine_create_layered(tm_engine** out, const tm_engine_config* c, const t
                                && !s.diff_maps && s.conv_taps == 0 && s.rot_dims == 0 && s.softcap <= 0.f,
                            at + ": left mixer: vdim = dim, kv_heads * dim <= 1024, dist_buckets >= 2, dist_max > dist_buckets / 2, no maps / convolution / rotation / cap");
                 TM_REQUIRE(s.r_heads >= 1 && s.r_kv_heads >= 1 && s.r_heads % s.r_kv_heads == 0 && s.r_dim >= 1 && s.r_dim <= 256 && s.r_vdim >= 1
-                               && s.r_vdim <= 1024 && s.r_conv >= 1 && s.r_conv <= 8 && s.a_rank >= 1 && s.g_rank >= 1,
-                           at + ": right mixer: r_heads % r_kv_heads, 1 <= r_dim <= 256, 1 <= r_vdim <= 1024, 1 <= r_conv <= 8, a_rank, g_rank >= 1");
+                               && s.r_vdim <= 1024 && s.r_conv >= 1 && s.r_conv <= 16 && s.a_rank >= 1 && s.g_rank >= 1,
+                           at + ": right mixer: r_heads % r_kv_heads, 1 <= r_dim <= 256, 1 <= r_vdim <= 1024, 1 <= r_conv <= 16, a_rank, g_rank >= 1");
             }
             continue;
         }

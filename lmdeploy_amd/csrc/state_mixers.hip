@@ -564,7 +564,7 @@ __global__ __launch_bounds__(256) void short_conv_kernel(float* __restrict__ y, 
 int launch_short_conv(float* y, int ldy, const float* x, int ldx, int x_col, const float* w, int channels, int taps, int act,
                       const StateMixParams& p, hipStream_t st)
 {
-    TM_REQUIRE(y && x && w && channels >= 1 && ldy >= channels && ldx >= x_col + channels && taps >= 1 && taps <= 8, "short conv: operands (1 <= taps <= 8)");
+    TM_REQUIRE(y && x && w && channels >= 1 && ldy >= channels && ldx >= x_col + channels && taps >= 1 && taps <= 16, "short conv: operands (1 <= taps <= 16)");
     TM_REQUIRE(p.cu_q && p.k_len && (taps == 1 || p.state) && p.max_q_len >= 1, "short conv: sequences / state");
     if (p.nseq == 0) {
         return 0;
@@ -573,8 +573,11 @@ int launch_short_conv(float* y, int ldy, const float* x, int ldx, int x_col, con
     if (taps <= 4) {
         short_conv_kernel<4><<<grid, 256, 0, st>>>(y, ldy, x, ldx, x_col, w, channels, taps, act, p);
     }
-    else {
+    else if (taps <= 8) {
         short_conv_kernel<8><<<grid, 256, 0, st>>>(y, ldy, x, ldx, x_col, w, channels, taps, act, p);
+    }
+    else {
+        short_conv_kernel<16><<<grid, 256, 0, st>>>(y, ldy, x, ldx, x_col, w, channels, taps, act, p);
     }
     TM_HIP_CHECK(hipGetLastError());
     return 0;
