@@ -365,6 +365,45 @@ def test_engine_long_decoding_far_beyond_the_windows(cuda, tmp_path, dtype):
     eng.close()
 
 
+@pytest.mark.parametrize('dtype', ['float32', 'bfloat16'])
+@pytest.mark.parametrize('kind', ['differential', 'left'])
+def test_window_edges_through_the_engine(cuda, tmp_path, dtype, kind):
+    """one-layer models whose only way back in time is the window (one-tap convolutions; the delta rule's branch weighs zero): another
+    token just outside a row's window leaves the row's logits as they are, another token at the window's last position moves them --
+    windows that end inside a block and on a block border, prompt rows and decoded rows"""
+    for W in (37, 64):
+        if kind == 'differential':
+            cfg = mo.make_config(48, 61, [mo.attention_layer(2, 1, 16, 16, 0.4, W, 8, 1000.0, None, 0.0, 0.4, 1)], groups=2)
+            w = mo.random_weights(cfg, 21)
+        else:
+            cfg = mo.make_config(48, 61, [mo.parallel_layer(mo.left_mixer(4, 2, 16, W, 50, 0.4), mo.right_mixer(2, 1, 8, 8, 2))], groups=2)
+            w = mo.random_weights(cfg, 21, buckets=8, a_rank=4, g_rank=4)
+            w['l0.mix.right.out'] = np.zeros_like(w['l0.mix.right.out'])
+        folder = str(tmp_path / f'{kind}{W}')
+        mo.write_checkpoint(folder, cfg, w)
+        eng = engine(folder, dtype)
+        toks = np.random.default_rng(W).integers(0, 61, 150).tolist()
+        rows = [W, 100, 128, 149]
+
+        def logits(t, decode_from):
+            s = eng.open_session()
+            out = eng.step_tokens([(s, t[:decode_from], [r for r in rows if r < decode_from])])
+            rest = [eng.step_tokens([(s, [x], [0])]) for x in t[decode_from:]]
+            eng.close_session(s)
+            return np.concatenate([out] + [rest[r - decode_from] for r in rows if r >= decode_from])
+
+        for decode_from in (150, 90):
+            base = logits(toks, decode_from)
+            assert rel_err(base, mo.forward(cfg, w, toks)[rows]) <= TOL[dtype]
+            for k, r in enumerate(rows):
+                for j, seen in ((r - W, False), (r - W + 1, True)):
+                    other = list(toks)
+                    other[j] = (toks[j] + 7) % 61
+                    moved = np.abs(logits(other, decode_from)[k] - base[k]).max() / base.std()
+                    assert (moved > 1e-3) == seen and (seen or moved <= 1e-6), (W, decode_from, r, j, moved)
+        eng.close()
+
+
 def test_state_of_a_far_token_survives_hundreds_of_steps(cuda, tmp_path):
     """a delta-rule state that barely decays (A_log far below zero) and writes weakly keeps a token from 300 positions back, far outside
     the left mixer's window: moving that one token moves the last logits, in one portion and when everything after the first portion is
