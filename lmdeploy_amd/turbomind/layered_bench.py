@@ -167,9 +167,9 @@ def mededra_config(s) -> dict:
     of 128, window 2048, scaled pairwise rotation, 4-tap convolutions.  Parallel pair: left = windowed attention over 2 key heads of 128
     (a wide key of 256) with the bucketed distance bias and mixed heads; right = gated delta rule with heads of 128 x 128"""
     b, H, G = MEDEDRA, s['heads'], s['kv_heads']
-    att = {'heads': H, 'kv_heads': G, 'dim': b['map_dim'], 'vdim': 128, 'scale': b['map_dim'] ** -0.5, 'softcap': 30.0, 'diff': 0.5, 'conv': b['conv'],
+    att = {'heads': H, 'kv_heads': G, 'dim': b['map_dim'], 'vdim': 128, 'scale': b['map_dim'] ** -0.5, 'softcap': 50.0, 'diff': 0.8, 'conv': b['conv'],
            'mask': {'size': b['window']},
-           'rot': {'base': 250000.0, 'dims': b['rot_dims'], 'scaling': {'factor': 8.0, 'original': 2048, 'fast': 32.0, 'slow': 1.0}}}
+           'rot': {'base': 1000000.0, 'dims': b['rot_dims'], 'scaling': {'factor': 4.0, 'original': 1024, 'fast': 16.0, 'slow': 2.0}}}
     left = {'heads': H, 'kv_heads': b['left_kv'], 'dim': 128, 'vdim': 128, 'scale': 128 ** -0.5, 'mask': {'size': b['window']},
             'bias_max': b['bias_max'], 'buckets': b['buckets']}
     right = {'heads': H, 'kv_heads': G, 'dim': 128, 'vdim': 128, 'conv': b['conv'], 'a_rank': b['rank'], 'g_rank': b['rank']}

@@ -75,10 +75,10 @@ def test_rotation_pairs_neighbours_and_scales_slow_frequencies():
 
 
 def test_distance_buckets():
-    B, D = 16, 240.0
-    assert [mo.distance_bucket(n, B, D) for n in range(8)] == list(range(8))
-    assert mo.distance_bucket(8, B, D) == 8 and mo.distance_bucket(12, B, D) == 8      # 8 ln(1.5) / ln(30) = 0.95
-    assert mo.distance_bucket(13, B, D) == 9 and mo.distance_bucket(239, B, D) == 15 and mo.distance_bucket(100000, B, D) == 15
+    B, D = 12, 100.0
+    assert [mo.distance_bucket(n, B, D) for n in range(6)] == list(range(6))
+    assert mo.distance_bucket(6, B, D) == 6 and mo.distance_bucket(9, B, D) == 6        # 6 ln(1.5) / ln(100 / 6) = 0.86
+    assert mo.distance_bucket(10, B, D) == 7 and mo.distance_bucket(99, B, D) == 11 and mo.distance_bucket(100000, B, D) == 11
     assert [mo.distance_bucket(n, 4, 8.0) for n in (0, 1, 2, 3, 4, 7, 8)] == [0, 1, 2, 2, 3, 3, 3]
 
 
