@@ -1064,6 +1064,9 @@ static int group_layer(tm_engine* e, const LmLayer& L, int M, const LmPart* part
     if (L.conv_taps > 0) {
         for (int i = 0; i < nparts; ++i) {
             const LmPart&  P  = parts[i];
+            if (P.decode && s.mixer == TM_MIXER_ATTENTION) {
+                continue;  // decoded tokens: the convolution runs inside the prepare kernel (one row per sequence)
+            }
             StateMixParams sp = state_seqs(e, P);
             sp.layer_offset   = L.conv_offset;
             TM_PROF(P_KV_STORE, TM_TRY(launch_short_conv(lm.d_conv + (size_t)P.row0 * lm.ldconv, lm.ldconv, lm.d_proj + (size_t)P.row0 * lm.ldproj, lm.ldproj,
@@ -1080,8 +1083,17 @@ static int group_layer(tm_engine* e, const LmLayer& L, int M, const LmPart* part
         for (int i = 0; i < nparts; ++i) {
             const LmPart&     P = parts[i];
             GeneralAttnParams p = attn_params(e, L, P);
-            TM_PROF(P_KV_STORE, TM_TRY(launch_attn_prep(src + (size_t)P.row0 * ld, ld, 0, L.c_k, L.c_v, (void*)p.q, lm.ldq, s.qk_norm_w != 0, false,
-                                                        m.norm_eps, p, st, ex)));
+            AttnPrepExtra     px = ex;
+            const bool        fused = P.decode && L.conv_taps > 0;
+            if (fused) {
+                px.conv_w = L.conv_w, px.conv_taps = L.conv_taps, px.conv_ch = L.conv_ch;
+                px.conv_state = lm.d_state, px.conv_slot_stride = lm.state_slot_floats, px.conv_offset = L.conv_offset;
+                px.conv_slot0 = P.slot0, px.conv_park_slot = e->cfg.max_batch_size, px.conv_active = P.active;
+            }
+            const float* from = fused ? lm.d_proj : src;
+            const int    ldf  = fused ? lm.ldproj : ld;
+            TM_PROF(P_KV_STORE, TM_TRY(launch_attn_prep(from + (size_t)P.row0 * ldf, ldf, 0, L.c_k, L.c_v, (void*)p.q, lm.ldq, s.qk_norm_w != 0, false,
+                                                        m.norm_eps, p, st, px)));
         }
         TM_TRY(run_attention_parts(e, L, parts, nparts));
         if (s.diff_maps) {

@@ -409,7 +409,38 @@ __global__ __launch_bounds__(256) void attn_prep_kernel(const float* __restrict_
     }
     const int    kind = u < H ? 0 : (u < H + G ? 1 : 2), src = kind == 0 ? u : (kind == 1 ? u - H : u - H - G);
     const int    n    = kind == 2 ? p.vdim : p.dim;
-    const float* x    = proj + (size_t)t * ld + (kind == 0 ? q_col : (kind == 1 ? k_col : v_col)) + (size_t)src * n;
+    const int    col0 = (kind == 0 ? q_col : (kind == 1 ? k_col : v_col)) + src * n;
+    const float* x    = proj + (size_t)t * ld + col0;
+    __shared__ float conv_out[4][256];
+    if (ex.conv_w) {  // one row per sequence: this wave owns the channels [col0, col0 + n) of the sequence's convolution state
+        const int sq = p.row_seq[t], ps = p.row_pos[t], nh = ex.conv_taps - 1, C = ex.conv_ch;
+        int       slot = p.seq_slot ? p.seq_slot[sq] : ex.conv_slot0 + sq;
+        if (ex.conv_active && !ex.conv_active[sq]) {
+            slot = ex.conv_park_slot;
+        }
+        float* st = ex.conv_state + (size_t)slot * ex.conv_slot_stride + ex.conv_offset;
+        for (int i = lane; i < n; i += 64) {
+            const int    ch = col0 + i;
+            const float* w  = ex.conv_w + (size_t)ch * ex.conv_taps;
+            const float  u  = x[i];
+            float        acc = 0.f;
+            for (int j = 0; j < nh; ++j) {
+                acc = fmaf(w[j], ps > 0 ? st[(size_t)j * C + ch] : 0.f, acc);
+            }
+            acc = fmaf(w[nh], u, acc);
+            for (int j = 0; j + 1 < nh; ++j) {
+                st[(size_t)j * C + ch] = ps > 0 ? st[(size_t)(j + 1) * C + ch] : 0.f;
+            }
+            if (nh > 0) {
+                st[(size_t)(nh - 1) * C + ch] = u;
+            }
+            conv_out[threadIdx.x >> 6][i] = acc;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        x = conv_out[threadIdx.x >> 6];
+    }
     // several maps per head leave map-major: source [head][map] -> head map * (heads / maps) + head
     const int maps = kind == 2 ? 1 : ex.maps, cnt = kind == 0 ? H : G;
     const int head = maps > 1 ? (src % maps) * (cnt / maps) + src / maps : src;
@@ -467,6 +498,8 @@ int launch_attn_prep(const float* proj, int ld, int q_col, int k_col, int v_col,
     TM_REQUIRE(ex.rot_dims >= 0 && ex.rot_dims % 2 == 0 && ex.rot_dims <= p.dim && (ex.rot_dims == 0 || ex.inv_freq), "attn_prep: rotation");
     const int kh = p.k_heads > 0 ? p.k_heads : p.kv_heads, vh = p.v_heads > 0 ? p.v_heads : p.kv_heads;
     TM_REQUIRE(ex.maps >= 1 && p.q_heads % ex.maps == 0 && kh % ex.maps == 0, "attn_prep: the maps divide the query and key heads");
+    TM_REQUIRE(!ex.conv_w || (p.dim <= 256 && p.vdim <= 256 && ex.conv_taps >= 1 && ex.conv_ch >= 1 && (ex.conv_taps == 1 || ex.conv_state)),
+               "attn_prep: fused convolution: head sizes up to 256, taps, channels, state");
     if (p.rows == 0) {
         return 0;
     }

@@ -475,6 +475,15 @@ struct AttnPrepExtra {
     int          rot_dims = 0;
     int          maps = 1, rot_pairs = 0;
     float        rot_mult = 1.f;
+    // conv_w != nullptr (launches with ONE row per sequence: decoded tokens): the source columns first pass the short causal convolution
+    // of launch_short_conv in this kernel -- column c is channel c of conv_w [conv_ch][conv_taps] and of the sequence's state
+    // [conv_taps - 1][conv_ch] at conv_state + slot * conv_slot_stride + conv_offset, which the wave that owns a channel reads and rewrites
+    const float* conv_w = nullptr;
+    int          conv_taps = 0, conv_ch = 0;
+    float*       conv_state = nullptr;
+    size_t       conv_slot_stride = 0, conv_offset = 0;
+    int          conv_slot0 = 0, conv_park_slot = 0;
+    const int*   conv_active = nullptr;
 };
 int launch_attn_prep(const float* proj, int ld, int q_col, int k_col, int v_col, void* q_out, int ldq, bool qk_norm, bool v_norm, float eps,
                      const GeneralAttnParams& layout, hipStream_t st, AttnPrepExtra extra = AttnPrepExtra());
